@@ -1,0 +1,158 @@
+"""CPU restatement of the reference's eager multi-head FFN.  TEST INFRASTRUCTURE ONLY.
+
+This file is the checker the HIP kernels are compared against; it is never the thing
+measured or shipped.  Every function cites the reference lines it restates.
+
+    forward, per (b, h, t), q = Q[b,h,t,:], expert e, kuv-head hk = h // G:
+        m_e = K[hk,e] q ; n_e = U[hk,e] q ; a_e = silu(m_e) * n_e ; o_e = V[hk,e]^T a_e
+        O[b,h,t,:] = sum_e R[b,h,t,e] * o_e
+
+Pinning status (what fixes each function independently of this file's own formulas):
+  * mhffn_forward            -- library routines (torch.matmul, F.silu); the E=1, R=1 case equals
+                                F.linear(silu(F.linear(q,K)) * F.linear(q,U), V^T); scalar C loops in
+                                oracle/mhffn_scalar.c; pure-Python brute force on tiny shapes.
+  * mhffn_backward (analytic)-- torch.autograd of mhffn_forward in fp64, torch.autograd.gradcheck,
+                                central finite differences, and the scalar C backward.
+  * tk_ground_truth          -- equals mhffn_forward up to rounding (same closed form).
+  * mhffn_layer_forward      -- library routines only (F.linear, sigmoid, sum).
+The reference holds no golden vectors for this path (it has no tests with stored data), so the
+vectors under tests/golden/ are produced by this oracle after it passed the checks above.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+
+def repeat_kuv(w: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """[H_kuv,E,d_e,d_h] -> [H_kuv*n_rep,E,d_e,d_h]; q-head i uses kuv-head i // n_rep.
+
+    Restates models/flashmhf/modeling_mhffnmoe.py:224-253 (the 4-D branch, :246-251).
+    """
+    if n_rep == 1:
+        return w
+    return torch.repeat_interleave(w, n_rep, dim=0)
+
+
+def mhffn_forward(Q, K, U, V, R, *, compute_dtype=None, out_dtype=None):
+    """Eager expert loop, models/flashmhf/modeling_mhffnmoe.py:412-431 with s0=s1=s2=1 (:270-279).
+
+    Q [B,H,S,d_h]; K,U,V [H_kuv,E,d_e,d_h]; R [B,H,S,E].  ``compute_dtype`` is the dtype the matmuls
+    and the activation run in (the reference runs them in x.dtype); each expert's result is cast to
+    fp32 (fp64 when compute_dtype is fp64) before the multiplication by R and the sum over experts
+    (:425), and the sum is cast to ``out_dtype`` at the end (:427).
+    """
+    compute_dtype = compute_dtype or Q.dtype
+    out_dtype = out_dtype or compute_dtype
+    acc_dtype = torch.float64 if compute_dtype == torch.float64 else torch.float32
+    H, Hk = Q.shape[1], K.shape[0]
+    assert H % Hk == 0
+    G = H // Hk
+    q = Q.to(compute_dtype)
+    k = repeat_kuv(K.to(compute_dtype), G)
+    u = repeat_kuv(U.to(compute_dtype), G)
+    v = repeat_kuv(V.to(compute_dtype), G)
+    r = R.to(acc_dtype)
+    out = torch.zeros(Q.shape, dtype=acc_dtype, device=Q.device)
+    for e in range(K.shape[1]):
+        w = q @ k[:, e].transpose(1, 2)                 # [B,H,S,d_e]   (:418)
+        w = F.silu(w)                                    # (:419)
+        w = w * (q @ u[:, e].transpose(1, 2))            # (:420)
+        out += (w @ v[:, e]).to(acc_dtype) * r[..., e:e + 1]   # (:425)
+    return out.to(out_dtype)
+
+
+def tk_ground_truth(Q, K, U, V, R):
+    """kernels/thunderkittens/run_from_python.py:19-24 -- the reference's own 5-line check (H == H_kuv)."""
+    O = torch.zeros_like(Q)
+    for e in range(K.shape[1]):
+        oi = (F.silu(Q @ K[:, e].transpose(1, 2)) * (Q @ U[:, e].transpose(1, 2))) @ V[:, e]
+        O = O + (oi * R[..., e:e + 1]).to(O.dtype)
+    return O
+
+
+def mhffn_backward(Q, K, U, V, R, dO, *, compute_dtype=torch.float64):
+    """Analytic backward, kernels/triton/flash_mlp_moe.py:401-414 extended by the R factor
+    (:534-536 for dR/dM/dN, :720-729 for dV/dK/dU).
+
+        dA = dO V^T ; dR_e = sum_j dA*silu(M)*N ; dN = R_e*dA*silu(M)
+        dM = R_e*dA*N*silu'(M), silu'(x) = sig(x) + x*sig(x)*(1-sig(x))      (:531)
+        dQ = sum_e dM K_e + dN U_e ; dK_e = dM^T Q ; dU_e = dN^T Q ; dV_e = (R_e*silu(M)*N)^T dO
+    dK/dU/dV are summed over batch, tokens and the G q-heads that share a kuv-head.
+    Returns (dQ, dK, dU, dV, dR) in ``compute_dtype``.
+    """
+    cd = compute_dtype
+    B, H, S, dh = Q.shape
+    Hk, E, de, _ = K.shape
+    G = H // Hk
+    q, g, r = Q.to(cd), dO.to(cd), R.to(cd)
+    k, u, v = (repeat_kuv(w.to(cd), G) for w in (K, U, V))
+    dQ = torch.zeros_like(q)
+    dK = torch.zeros((H, E, de, dh), dtype=cd)
+    dU = torch.zeros_like(dK)
+    dV = torch.zeros_like(dK)
+    dR = torch.zeros_like(r)
+    for e in range(E):
+        m = q @ k[:, e].transpose(1, 2)
+        n = q @ u[:, e].transpose(1, 2)
+        sig = torch.sigmoid(m)
+        s = m * sig
+        dA = g @ v[:, e].transpose(1, 2)
+        re = r[..., e:e + 1]
+        dR[..., e] = (dA * s * n).sum(-1)
+        dN = re * dA * s
+        dM = re * dA * n * (sig + s * (1 - sig))
+        dQ += dM @ k[:, e] + dN @ u[:, e]
+        dK[:, e] = (dM.transpose(2, 3) @ q).sum(0)
+        dU[:, e] = (dN.transpose(2, 3) @ q).sum(0)
+        dV[:, e] = ((re * s * n).transpose(2, 3) @ g).sum(0)
+    fold = lambda w: w.view(Hk, G, E, de, dh).sum(1)
+    return dQ, fold(dK), fold(dU), fold(dV), dR
+
+
+def mhffn_autograd(Q, K, U, V, R, dO, *, compute_dtype=torch.float64):
+    """Gradients of mhffn_forward by torch.autograd (the cross-check for mhffn_backward)."""
+    leaves = [t.detach().to(compute_dtype).requires_grad_(True) for t in (Q, K, U, V, R)]
+    out = mhffn_forward(*leaves, compute_dtype=compute_dtype)
+    grads = torch.autograd.grad(out, leaves, dO.to(out.dtype))
+    return out.detach(), grads
+
+
+def router_gate(Qh, router):
+    """R = sigmoid(Q.float() @ router.float()), divided by its sum over experts clamped at 1e-20.
+    models/flashmhf/modeling_mhffnmoe.py:384-386.  Qh [B,H,S,d_h], router [d_h,E] or [H,d_h,E]."""
+    R = (Qh.to(torch.float32) @ router.to(torch.float32)).contiguous().sigmoid()
+    return R / R.sum(dim=-1, keepdim=True).clamp(min=1e-20)
+
+
+def mhffn_layer_forward(X, Wq, Wr, K, U, V, Wo, *, num_heads, compute_dtype=torch.float32):
+    """The benchmark's CPU layer: Q = X Wq split into heads, R = sigmoid(X Wr) normalised over E,
+    the eager expert loop, heads merged, output projection Wo.
+
+    Follows models/flashmhf/modeling_mhffnmoe.py:352-431 with RMSNorm off (the 128M config) and the gate
+    logits taken from X through Wr [hid, H*E] as the benchmark configuration states.
+    X [B,S,hid]; Wq, Wo [hid,hid] used as x @ W.
+    """
+    B, S, hid = X.shape
+    H = num_heads
+    E = K.shape[1]
+    x = X.to(compute_dtype)
+    Qh = (x @ Wq.to(compute_dtype)).view(B, S, H, hid // H).transpose(1, 2).contiguous()
+    Rl = (X.to(torch.float32) @ Wr.to(torch.float32)).view(B, S, H, E).transpose(1, 2).sigmoid()
+    R = (Rl / Rl.sum(-1, keepdim=True).clamp(min=1e-20)).contiguous()
+    Oh = mhffn_forward(Qh, K, U, V, R, compute_dtype=compute_dtype)
+    O = Oh.transpose(1, 2).contiguous().view(B, S, hid)
+    return O @ Wo.to(compute_dtype), Qh, R, Oh
+
+
+def error_metrics(x, ref):
+    """max-abs, max-abs normalised by max|ref| (kernels/thunderkittens/run_from_python.py:54-58 prints this
+    as a percentage) and mean relative error sum|x-ref| / sum|ref|."""
+    x = x.detach().double().cpu()
+    ref = ref.detach().double().cpu()
+    d = (x - ref).abs()
+    return {
+        "max_abs": d.max().item(),
+        "norm_max": (d.max() / ref.abs().max().clamp(min=1e-30)).item(),
+        "mean_rel": (d.sum() / ref.abs().sum().clamp(min=1e-30)).item(),
+    }

@@ -1,0 +1,161 @@
+"""Pins the CPU oracle without the reference: library routines, brute force, autograd, finite differences,
+closed-form special cases and invariants.  Each check is chosen so that a dropped term, a wrong sign, a wrong
+index or a transposed operand fails it."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import mhffn_oracle as orc
+from tests.helpers import make_inputs
+
+D = torch.float64
+
+
+def _tiny(seed=0, **kw):
+    shape = dict(B=2, H=4, S=5, dh=6, E=3, de=7, Hk=2)
+    shape.update(kw)
+    return make_inputs(**shape, seed=seed, dtype=D, r_mode="randn")
+
+
+def test_forward_matches_pure_python_brute_force():
+    Q, K, U, V, R, _ = make_inputs(1, 1, 3, 4, 2, 3, seed=1, dtype=D, r_mode="randn")
+    O = orc.mhffn_forward(Q, K, U, V, R)
+    for t in range(3):
+        for c in range(4):
+            acc = 0.0
+            for e in range(2):
+                for j in range(3):
+                    m = sum(Q[0, 0, t, x].item() * K[0, e, j, x].item() for x in range(4))
+                    n = sum(Q[0, 0, t, x].item() * U[0, e, j, x].item() for x in range(4))
+                    acc += R[0, 0, t, e].item() * (m / (1 + math.exp(-m))) * n * V[0, e, j, c].item()
+            assert abs(O[0, 0, t, c].item() - acc) < 1e-12
+
+
+def test_forward_and_backward_match_scalar_c(scalar_oracle):
+    Q, K, U, V, R, dO = _tiny(seed=2)
+    O = orc.mhffn_forward(Q, K, U, V, R)
+    O_c = scalar_oracle.forward(*(t.numpy() for t in (Q, K, U, V, R)))
+    np.testing.assert_allclose(O.numpy(), O_c, rtol=0, atol=1e-12)
+    grads = orc.mhffn_backward(Q, K, U, V, R, dO)
+    grads_c = scalar_oracle.backward(*(t.numpy() for t in (Q, K, U, V, R, dO)))
+    for g, gc in zip(grads, grads_c):
+        np.testing.assert_allclose(g.numpy(), gc, rtol=0, atol=1e-11)
+
+
+def test_analytic_backward_matches_autograd():
+    Q, K, U, V, R, dO = _tiny(seed=3)
+    _, auto = orc.mhffn_autograd(Q, K, U, V, R, dO)
+    ana = orc.mhffn_backward(Q, K, U, V, R, dO)
+    for a, b in zip(ana, auto):
+        assert (a - b).abs().max().item() < 1e-11
+
+
+def test_gradcheck_fp64():
+    Q, K, U, V, R, _ = make_inputs(1, 2, 3, 4, 2, 3, Hk=1, seed=4, dtype=D, r_mode="randn")
+    leaves = [t.clone().requires_grad_(True) for t in (Q, K, U, V, R)]
+    assert torch.autograd.gradcheck(lambda *a: orc.mhffn_forward(*a, compute_dtype=D), leaves, eps=1e-6, atol=1e-6)
+
+
+def test_backward_central_differences():
+    Q, K, U, V, R, dO = make_inputs(1, 2, 3, 4, 2, 3, Hk=2, seed=5, dtype=D, r_mode="randn")
+    dQ, dK, dU, dV, dR = orc.mhffn_backward(Q, K, U, V, R, dO)
+    loss = lambda *a: (orc.mhffn_forward(*a) * dO).sum().item()
+    args = [Q, K, U, V, R]
+    for idx, grad in enumerate((dQ, dK, dU, dV, dR)):
+        flat = args[idx].reshape(-1)
+        for pos in range(0, flat.numel(), max(1, flat.numel() // 7)):
+            old = flat[pos].item()
+            flat[pos] = old + 1e-6
+            lp = loss(*args)
+            flat[pos] = old - 1e-6
+            lm = loss(*args)
+            flat[pos] = old
+            assert abs((lp - lm) / 2e-6 - grad.reshape(-1)[pos].item()) < 1e-6
+
+
+def test_single_expert_unit_gate_is_per_head_swiglu():
+    """E=1, R=1: O_h = down_h(silu(gate_h(q)) * up_h(q)) with F.linear (legacy kernels/triton/flash_mlp.py:153-156)."""
+    Q, K, U, V, _, _ = make_inputs(2, 3, 5, 8, 1, 16, seed=6, dtype=D)
+    R = torch.ones(2, 3, 5, 1, dtype=D)
+    O = orc.mhffn_forward(Q, K, U, V, R)
+    for h in range(3):
+        ref = F.linear(F.silu(F.linear(Q[:, h], K[h, 0])) * F.linear(Q[:, h], U[h, 0]), V[h, 0].t())
+        assert (O[:, h] - ref).abs().max().item() < 1e-12
+
+
+def test_constant_gate_equals_one_wide_expert():
+    Q, K, U, V, _, _ = _tiny(seed=7, Hk=4)
+    c = 0.37
+    R = torch.full((2, 4, 5, 3), c, dtype=D)
+    O = orc.mhffn_forward(Q, K, U, V, R)
+    wide = lambda w: w.reshape(4, 1, 21, 6)
+    O1 = orc.mhffn_forward(Q, wide(K), wide(U), wide(V), torch.full((2, 4, 5, 1), c, dtype=D))
+    assert (O - O1).abs().max().item() < 1e-12
+
+
+def test_linearity_zero_and_permutation_invariants():
+    Q, K, U, V, R, dO = _tiny(seed=8)
+    O = orc.mhffn_forward(Q, K, U, V, R)
+    assert (orc.mhffn_forward(Q, K, U, V, -2.5 * R) + 2.5 * O).abs().max().item() < 1e-12
+    V2 = torch.randn_like(V)
+    assert (orc.mhffn_forward(Q, K, U, V + V2, R) - O - orc.mhffn_forward(Q, K, U, V2, R)).abs().max().item() < 1e-12
+    assert orc.mhffn_forward(Q, K * 0, U, V, R).abs().max().item() == 0
+    assert orc.mhffn_forward(Q, K, U * 0, V, R).abs().max().item() == 0
+    pj = torch.randperm(7)
+    pe = torch.randperm(3)
+    Op = orc.mhffn_forward(Q, K[:, pe][:, :, pj], U[:, pe][:, :, pj], V[:, pe][:, :, pj], R[..., pe])
+    assert (Op - O).abs().max().item() < 1e-12
+    pt = torch.randperm(5)
+    assert (orc.mhffn_forward(Q[:, :, pt], K, U, V, R[:, :, pt]) - O[:, :, pt]).abs().max().item() < 1e-12
+
+
+def test_dR_is_inner_product_with_per_expert_output():
+    Q, K, U, V, R, dO = _tiny(seed=9)
+    dR = orc.mhffn_backward(Q, K, U, V, R, dO)[4]
+    for e in range(3):
+        onehot = torch.zeros_like(R)
+        onehot[..., e] = 1
+        Oe = orc.mhffn_forward(Q, K, U, V, onehot)
+        assert ((Oe * dO).sum(-1) - dR[..., e]).abs().max().item() < 1e-11
+
+
+def test_grouped_kuv_heads_use_integer_division():
+    Q, K, U, V, R, _ = _tiny(seed=10)          # H=4, Hk=2 -> q-heads 0,1 share kuv-head 0
+    O = orc.mhffn_forward(Q, K, U, V, R)
+    for h in range(4):
+        Oh = orc.mhffn_forward(Q[:, h:h + 1], K[h // 2:h // 2 + 1], U[h // 2:h // 2 + 1], V[h // 2:h // 2 + 1], R[:, h:h + 1])
+        assert (O[:, h:h + 1] - Oh).abs().max().item() < 1e-12
+
+
+def test_tk_ground_truth_agrees_with_eager_loop():
+    Q, K, U, V, R, _ = _tiny(seed=11, Hk=4)
+    assert (orc.tk_ground_truth(Q, K, U, V, R) - orc.mhffn_forward(Q, K, U, V, R)).abs().max().item() < 1e-12
+
+
+def test_router_gate_rows_sum_to_one_and_layer_shapes():
+    g = torch.Generator().manual_seed(12)
+    B, S, hid, H, E, de = 2, 4, 24, 4, 3, 8
+    X = torch.randn(B, S, hid, generator=g)
+    Wq, Wo = torch.randn(hid, hid, generator=g) / hid ** 0.5, torch.randn(hid, hid, generator=g) / hid ** 0.5
+    Wr = torch.randn(hid, H * E, generator=g) * 0.02
+    K, U, V = (torch.randn(H, E, de, hid // H, generator=g) for _ in range(3))
+    Y, Qh, R, Oh = orc.mhffn_layer_forward(X, Wq, Wr, K, U, V, Wo, num_heads=H)
+    assert Y.shape == (B, S, hid) and Qh.shape == (B, H, S, hid // H) and R.shape == (B, H, S, E)
+    assert (R.sum(-1) - 1).abs().max().item() < 1e-6
+    # head h of Qh is columns [h*dh,(h+1)*dh) of X@Wq
+    assert (Qh[:, 1] - (X @ Wq)[..., 6:12]).abs().max().item() < 1e-6
+    Rg = orc.router_gate(Qh, torch.randn(hid // H, E, generator=g))
+    assert (Rg.sum(-1) - 1).abs().max().item() < 1e-6
+
+
+def test_bf16_eager_is_within_tolerance_of_fp32_oracle():
+    """The reference's own bf16 eager path vs the fp32 oracle on the same rounded inputs: documents that the
+    2e-2 / 1e-2 bar is meaningful for the benchmark distributions."""
+    Q, K, U, V, R, _ = make_inputs(1, 2, 64, 96, 8, 256, seed=13, dtype=torch.bfloat16)
+    ref = orc.mhffn_forward(Q, K, U, V, R, compute_dtype=torch.float32)
+    got = orc.mhffn_forward(Q, K, U, V, R, compute_dtype=torch.bfloat16, out_dtype=torch.float32)
+    m = orc.error_metrics(got, ref)
+    assert m["max_abs"] < 2e-2 and m["mean_rel"] < 1e-2
