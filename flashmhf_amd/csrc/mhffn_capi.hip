@@ -1,0 +1,99 @@
+// C ABI of libmhffn_hip.so: argument validation, error codes, dispatch.  No torch, no pybind, no allocation.
+#include "../../include/mhffn.h"
+#include "mhffn_common.hpp"
+
+namespace {
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_dims_impl(const mhffn_dims* d, int dtype)
+{
+    if (!d) return MHFFN_ERR_NULL_POINTER;
+    if (dtype != MHFFN_DTYPE_BF16 && dtype != MHFFN_DTYPE_F32) return MHFFN_ERR_DTYPE;
+    if (d->B <= 0 || d->H <= 0 || d->Hkuv <= 0 || d->S <= 0 || d->E <= 0 || d->d_e <= 0 || d->d_h <= 0)
+        return MHFFN_ERR_SHAPE;
+    if (d->H % d->Hkuv != 0) return MHFFN_ERR_SHAPE;
+    if (dtype == MHFFN_DTYPE_F32) return MHFFN_ERR_DTYPE;   // no fp32 kernels in this build
+    if (d->d_h != 64 && d->d_h != 96 && d->d_h != 128) return MHFFN_ERR_HEAD_DIM;
+    if (d->d_e % 32 != 0) return MHFFN_ERR_EXPERT_DIM;
+    // index arithmetic inside the kernels is 64-bit for rows, 32-bit for per-(b,h) token indices and grid extents
+    if ((long long)d->B > 65535 || (long long)d->S > (1ll << 30)) return MHFFN_ERR_SHAPE;
+    return MHFFN_OK;
+}
+
+mhffn::Dims to_dims(const mhffn_dims* d) { return mhffn::Dims{d->B, d->H, d->Hkuv, d->S, d->d_h, d->E, d->d_e}; }
+
+}  // namespace
+
+extern "C" {
+
+const char* mhffn_strerror(int code)
+{
+    switch (code) {
+        case MHFFN_OK: return "ok";
+        case MHFFN_ERR_NULL_POINTER: return "null pointer argument";
+        case MHFFN_ERR_DTYPE: return "unsupported dtype (Q, K, U, V must be bfloat16; R float32)";
+        case MHFFN_ERR_HEAD_DIM: return "unsupported head dim (d_h must be 64, 96 or 128)";
+        case MHFFN_ERR_EXPERT_DIM: return "unsupported expert dim (d_e must be a multiple of 32)";
+        case MHFFN_ERR_SHAPE: return "invalid extents (all must be positive, H a multiple of Hkuv)";
+        case MHFFN_ERR_WORKSPACE: return "workspace missing or too small";
+        case MHFFN_ERR_LAUNCH: return "kernel launch failed";
+        case MHFFN_ERR_ALIGNMENT: return "pointer not 16-byte aligned";
+    }
+    return "unknown error code";
+}
+
+int mhffn_is_supported(int d_h, int d_e, int dtype)
+{
+    if (dtype != MHFFN_DTYPE_BF16) return 0;
+    return (d_h == 64 || d_h == 96 || d_h == 128) && d_e > 0 && d_e % 32 == 0;
+}
+
+int mhffn_check_dims(const mhffn_dims* dims, int dtype) { return check_dims_impl(dims, dtype); }
+
+size_t mhffn_fwd_workspace_bytes(const mhffn_dims* dims, int dtype)
+{
+    if (check_dims_impl(dims, dtype) != MHFFN_OK) return 0;
+    return mhffn::fwd_workspace_bytes_bf16(to_dims(dims));
+}
+
+size_t mhffn_bwd_workspace_bytes(const mhffn_dims* dims, int dtype)
+{
+    if (check_dims_impl(dims, dtype) != MHFFN_OK) return 0;
+    return mhffn::bwd_workspace_bytes_bf16(to_dims(dims));
+}
+
+int mhffn_fwd(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
+              void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream)
+{
+    const int rc = check_dims_impl(dims, dtype);
+    if (rc != MHFFN_OK) return rc;
+    if (!Q || !K || !U || !V || !R || !O) return MHFFN_ERR_NULL_POINTER;
+    if (!aligned16(Q) || !aligned16(K) || !aligned16(U) || !aligned16(V) || !aligned16(R) || !aligned16(O) ||
+        !aligned16(workspace))
+        return MHFFN_ERR_ALIGNMENT;
+    const mhffn::Dims d = to_dims(dims);
+    if (!workspace || workspace_bytes < mhffn::fwd_workspace_bytes_bf16(d)) return MHFFN_ERR_WORKSPACE;
+    const hipError_t err = mhffn::launch_fwd_bf16(Q, K, U, V, R, O, workspace, d, (hipStream_t)stream);
+    return err == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
+}
+
+int mhffn_bwd(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
+              void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_dtype,
+              void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream)
+{
+    const int rc = check_dims_impl(dims, dtype);
+    if (rc != MHFFN_OK) return rc;
+    if (grad_w_dtype != MHFFN_DTYPE_BF16 && grad_w_dtype != MHFFN_DTYPE_F32) return MHFFN_ERR_DTYPE;
+    if (!Q || !K || !U || !V || !R || !dO || !dQ || !dK || !dU || !dV || !dR) return MHFFN_ERR_NULL_POINTER;
+    const void* ptrs[] = {Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, workspace};
+    for (const void* p : ptrs)
+        if (!aligned16(p)) return MHFFN_ERR_ALIGNMENT;
+    const mhffn::Dims d = to_dims(dims);
+    if (!workspace || workspace_bytes < mhffn::bwd_workspace_bytes_bf16(d)) return MHFFN_ERR_WORKSPACE;
+    const hipError_t err = mhffn::launch_bwd_bf16(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR,
+                                                  grad_w_dtype == MHFFN_DTYPE_F32, workspace, d, (hipStream_t)stream);
+    return err == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
+}
+
+}  // extern "C"

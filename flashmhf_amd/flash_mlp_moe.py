@@ -1,0 +1,116 @@
+"""Drop-in for the reference's ``kernels/triton/flash_mlp_moe.py`` operator boundary
+(``FlashMLPFunction`` :739-868, ``FlashMLPMoE`` :871-903), backed by hand-written gfx950 HIP kernels.
+
+    from flashmhf_amd.flash_mlp_moe import FlashMLPMoE
+    O = FlashMLPMoE()(Q, K, U, V, R)      # Q [B,H,S,d_h] bf16; K,U,V [Hkuv,E,d_e,d_h] bf16; R [B,H,S,E] fp32
+
+Same call signature, tensor contract, saved tensors (Q, K, U, V, R only -- no activations) and exception types.
+Differences, all widening: d_e may be any multiple of 32 (the reference needs 64, :758), the sequence length is
+free, and R's gradient is exact fp32 instead of bf16-rounded (:542).
+"""
+import torch
+
+from . import _capi
+
+
+def _dims(Q, K):
+    B, H, S, dh = Q.shape
+    Hk, E, de, dh2 = K.shape
+    if dh2 != dh:
+        raise RuntimeError(f"head dim mismatch: Q has {dh}, K has {dh2}")
+    return _capi.Dims(B, H, Hk, S, dh, E, de)
+
+
+def _check_inputs(Q, K, U, V, R):
+    if Q.dim() != 4 or K.dim() != 4 or R.dim() != 4:
+        raise RuntimeError("expected Q [B,H,S,d_h], K/U/V [Hkuv,E,d_e,d_h], R [B,H,S,E]")
+    expected = torch.bfloat16
+    if Q.dtype != expected or K.dtype != expected or V.dtype != expected or U.dtype != expected:
+        raise TypeError(
+            f"FlashMLPFunction expects all inputs in {expected}, got Q={Q.dtype}, K={K.dtype}, V={V.dtype}, U={U.dtype}")
+    if R.dtype != torch.float32:
+        raise TypeError(f"R must be float32 (the router gate is computed in fp32), got {R.dtype}")
+    if U.shape != K.shape or V.shape != K.shape:
+        raise RuntimeError(f"K, U, V must share one shape, got {tuple(K.shape)}, {tuple(U.shape)}, {tuple(V.shape)}")
+    if R.shape != (*Q.shape[:3], K.shape[1]):
+        raise RuntimeError(f"R must be [B,H,S,E] = {(*Q.shape[:3], K.shape[1])}, got {tuple(R.shape)}")
+    if K.shape[2] % 32 != 0:
+        raise ValueError(f"Expert dimension {K.shape[2]} must be divisible by 32")
+    if not Q.is_cuda:
+        raise RuntimeError("flashmhf_amd runs on the GPU only; there is no CPU path")
+    for name, t in (("Q", Q), ("K", K), ("U", U), ("V", V), ("R", R)):
+        if t.device != Q.device:
+            raise RuntimeError(f"{name} is on {t.device}, Q on {Q.device}")
+
+
+def _ws(nbytes, device):
+    return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)
+
+
+def mhffn_forward(Q, K, U, V, R):
+    """Launches the fused forward on the current stream and returns O (same shape and dtype as Q)."""
+    _check_inputs(Q, K, U, V, R)
+    Q, K, U, V, R = (t.contiguous() for t in (Q, K, U, V, R))
+    L = _capi.lib()
+    dims = _dims(Q, K)
+    code = _capi.torch_dtype_code(Q.dtype)
+    _capi.raise_for_code(L.mhffn_check_dims(dims, code), "mhffn_fwd")
+    O = torch.empty_like(Q)
+    nbytes = L.mhffn_fwd_workspace_bytes(dims, code)
+    ws = _ws(nbytes, Q.device)
+    with torch.cuda.device(Q.device):
+        rc = L.mhffn_fwd(Q.data_ptr(), K.data_ptr(), U.data_ptr(), V.data_ptr(), R.data_ptr(), O.data_ptr(),
+                         ws.data_ptr(), ws.numel(), dims, code, torch.cuda.current_stream().cuda_stream)
+    _capi.raise_for_code(rc, "mhffn_fwd")
+    return O
+
+
+def mhffn_backward(Q, K, U, V, R, dO, grad_w_dtype=torch.bfloat16):
+    """Launches the fused backward; returns (dQ, dK, dU, dV, dR).  dQ has Q's dtype, dR is fp32,
+    dK/dU/dV have ``grad_w_dtype`` (bf16 as flash_mlp_moe.py:808-810, or fp32 as flash_ffn_moe_torch.py:18-20)."""
+    _check_inputs(Q, K, U, V, R)
+    assert dO.shape == Q.shape, "grad_output shape should be the same as Q"
+    Q, K, U, V, R = (t.contiguous() for t in (Q, K, U, V, R))
+    dO = dO.to(Q.dtype).contiguous()
+    L = _capi.lib()
+    dims = _dims(Q, K)
+    code = _capi.torch_dtype_code(Q.dtype)
+    _capi.raise_for_code(L.mhffn_check_dims(dims, code), "mhffn_bwd")
+    dQ = torch.empty_like(Q)
+    dK, dU, dV = (torch.empty(K.shape, dtype=grad_w_dtype, device=K.device) for _ in range(3))
+    dR = torch.empty_like(R)
+    ws = _ws(L.mhffn_bwd_workspace_bytes(dims, code), Q.device)
+    with torch.cuda.device(Q.device):
+        rc = L.mhffn_bwd(Q.data_ptr(), K.data_ptr(), U.data_ptr(), V.data_ptr(), R.data_ptr(), dO.data_ptr(),
+                         dQ.data_ptr(), dK.data_ptr(), dU.data_ptr(), dV.data_ptr(), dR.data_ptr(),
+                         _capi.torch_dtype_code(grad_w_dtype), ws.data_ptr(), ws.numel(), dims, code,
+                         torch.cuda.current_stream().cuda_stream)
+    _capi.raise_for_code(rc, "mhffn_bwd")
+    return dQ, dK, dU, dV, dR
+
+
+class FlashMLPFunction(torch.autograd.Function):
+    """forward(ctx, Q, K, U, V, R) -> O ; backward(ctx, dO) -> (dQ, dK, dU, dV, dR).
+    Mirrors kernels/triton/flash_mlp_moe.py:739-868."""
+
+    @staticmethod
+    def forward(ctx, Q, K, U, V, R):
+        O = mhffn_forward(Q, K, U, V, R)
+        ctx.save_for_backward(Q, K, U, V, R)
+        return O
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        Q, K, U, V, R = ctx.saved_tensors
+        assert grad_output.shape == Q.shape, "grad_output shape should be the same as Q"
+        return mhffn_backward(Q, K, U, V, R, grad_output, grad_w_dtype=K.dtype)
+
+
+class FlashMLPMoE(torch.nn.Module):
+    """Stateless module, ``forward(Q, K, U, V, R) -> O``.  Mirrors kernels/triton/flash_mlp_moe.py:871-903."""
+
+    def __init__(self):
+        super().__init__()
+
+    def forward(self, Q, K, U, V, R):
+        return FlashMLPFunction.apply(Q, K, U, V, R)

@@ -1,0 +1,96 @@
+/* C ABI of the MI355X (gfx950) fused multi-head FFN library, libmhffn_hip.so.
+ *
+ *   O[b,h,t,:] = sum_e R[b,h,t,e] * ( (silu(Q[b,h,t,:] K[hk,e]^T) * (Q[b,h,t,:] U[hk,e]^T)) V[hk,e] ),   hk = h / (H/Hkuv)
+ *
+ * These entry points are what the reference's Python operator boundary binds for this path:
+ *   - kernels/triton/flash_mlp_moe.py:739-868   FlashMLPFunction.forward / .backward (Triton launches)
+ *   - kernels/thunderkittens/flash_ffn_moe.cu:938-1007, 1012-1133  flashffn_moe_forward / flashffn_moe_backward
+ *     (the pybind11 launchers, exported at :1135-1138)
+ *
+ * Conventions for every call:
+ *   - all tensor pointers are DEVICE pointers to contiguous row-major buffers owned by the caller, 16-byte aligned:
+ *       Q, O, dO, dQ   [B, H, S, d_h]
+ *       K, U, V        [Hkuv, E, d_e, d_h]        dK, dU, dV same shape
+ *       R, dR          [B, H, S, E]   always float32 (models/flashmhf/modeling_mhffnmoe.py:384-386)
+ *   - `dtype` is the element type of Q, K, U, V, O, dO, dQ (MHFFN_DTYPE_*).
+ *   - the library never allocates, never synchronises and never throws; work is enqueued on `stream`
+ *     (a hipStream_t passed as void*, NULL = the default stream).
+ *   - return value: MHFFN_OK or a negative MHFFN_ERR_* code; all argument checks happen before any launch.
+ *   - `workspace` is caller-provided device scratch of at least the size the matching *_workspace_bytes()
+ *     call reports (16-byte aligned).  Its contents are undefined after the call.
+ */
+#ifndef MHFFN_H_
+#define MHFFN_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    MHFFN_DTYPE_BF16 = 0,
+    MHFFN_DTYPE_F32  = 1
+};
+
+enum {
+    MHFFN_OK               =  0,
+    MHFFN_ERR_NULL_POINTER = -1,
+    MHFFN_ERR_DTYPE        = -2,  /* reference: TypeError, flash_mlp_moe.py:761-766; TORCH_CHECK flash_ffn_moe.cu:943-945 */
+    MHFFN_ERR_HEAD_DIM     = -3,  /* reference: assert head_dim == 128, flash_ffn_moe.cu:956 */
+    MHFFN_ERR_EXPERT_DIM   = -4,  /* reference: ValueError, flash_mlp_moe.py:758-759; assert flash_ffn_moe.cu:958 */
+    MHFFN_ERR_SHAPE        = -5,  /* non-positive extent, H not a multiple of Hkuv */
+    MHFFN_ERR_WORKSPACE    = -6,  /* workspace missing or smaller than *_workspace_bytes() */
+    MHFFN_ERR_LAUNCH       = -7,  /* hipGetLastError() after a launch */
+    MHFFN_ERR_ALIGNMENT    = -8   /* a tensor or workspace pointer is not 16-byte aligned */
+};
+
+/* Problem extents, shared by every call. */
+typedef struct mhffn_dims {
+    int B;      /* batch */
+    int H;      /* q heads */
+    int Hkuv;   /* K/U/V heads; H % Hkuv == 0 (grouped "GQ-FFN", flash_mlp_moe.py:194,222) */
+    int S;      /* tokens per (batch, head) */
+    int d_h;    /* head dim */
+    int E;      /* experts (sub-networks) per head */
+    int d_e;    /* rows of K/U/V per expert */
+} mhffn_dims;
+
+/* Human-readable text for a return code (static storage). */
+const char* mhffn_strerror(int code);
+
+/* 1 if kernels exist for (d_h, d_e, dtype), else 0.  bf16: d_h in {64, 96, 128}, d_e % 32 == 0.
+ * Replaces the reference's shape gates (flash_mlp_moe.py:758, flash_ffn_moe.cu:956-958, 1037). */
+int mhffn_is_supported(int d_h, int d_e, int dtype);
+
+/* Checks extents and dtype only (no pointers, no GPU).  Returns MHFFN_OK or the error the launch would return. */
+int mhffn_check_dims(const mhffn_dims* dims, int dtype);
+
+/* Scratch bytes needed by mhffn_fwd / mhffn_bwd for these extents (0 on invalid extents). */
+size_t mhffn_fwd_workspace_bytes(const mhffn_dims* dims, int dtype);
+size_t mhffn_bwd_workspace_bytes(const mhffn_dims* dims, int dtype);
+
+/* Forward.  Replaces the launch in FlashMLPFunction.forward (flash_mlp_moe.py:777-790) and
+ * flashffn_moe_forward (flash_ffn_moe.cu:938-1007).  O is written, nothing else. */
+int mhffn_fwd(const void* Q, const void* K, const void* U, const void* V, const float* R,
+              void* O,
+              void* workspace, size_t workspace_bytes,
+              const mhffn_dims* dims, int dtype, void* stream);
+
+/* Backward.  Replaces the two launches in FlashMLPFunction.backward (flash_mlp_moe.py:832-866) and
+ * flashffn_moe_backward (flash_ffn_moe.cu:1012-1133).
+ *   dQ has `dtype`; dR is float32 (flash_mlp_moe.py:811).
+ *   dK, dU, dV have `grad_w_dtype`: MHFFN_DTYPE_BF16 as the Triton wrapper allocates them
+ *   (flash_mlp_moe.py:808-810) or MHFFN_DTYPE_F32 as the ThunderKittens wrapper does
+ *   (flash_ffn_moe_torch.py:18-20).  They are overwritten (no need to zero them first). */
+int mhffn_bwd(const void* Q, const void* K, const void* U, const void* V, const float* R,
+              const void* dO,
+              void* dQ, void* dK, void* dU, void* dV, float* dR,
+              int grad_w_dtype,
+              void* workspace, size_t workspace_bytes,
+              const mhffn_dims* dims, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MHFFN_H_ */
