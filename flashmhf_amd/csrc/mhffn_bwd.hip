@@ -440,15 +440,18 @@ size_t bwd_workspace_bytes_bf16(const Dims& d)
 template <int DH>
 static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, const void* V, const float* R,
                                const void* dO, void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32,
-                               void* ws, const Dims& d, hipStream_t st)
+                               void* ws, const Dims& d, hipStream_t st, int phases)
 {
     constexpr int NCT = 2;
-    hipError_t err = launch_pack_weights(K, U, V, ws, 1, d, st);
-    if (err != hipSuccess) return err;
+    hipError_t err = hipSuccess;
+    if (phases & 1) {
+        err = launch_pack_weights(K, U, V, ws, 1, d, st);
+        if (err != hipSuccess) return err;
+    }
     float* part = reinterpret_cast<float*>((char*)ws + align256(packed_weights_bytes(d, 1)));
     const int nbe = d.d_e / JB, G = d.H / d.Hkuv;
 
-    {
+    if (phases & 2) {
         DqArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)ws, R, (bf16_t*)dQ, dR, d.H, G, d.S, d.E, nbe};
         constexpr int smem = 2 * Geo<DH>::DQ_STAGE * (int)sizeof(bf16_t);
         static bool attr_done = false;   // raising the dynamic LDS limit is a per-process, per-kernel property
@@ -464,8 +467,8 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }
-    {
-        const int nslice = pick_nslice(d);
+    const int nslice = pick_nslice(d);
+    if (phases & 4) {
         DwArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, part,
                  d.B, d.H, G, d.S, d.E, nbe, nslice};
         const int smem = 2 * (2 * Geo<DH>::NAT_ELEMS * 2 + d.E * 36 * 4);
@@ -475,6 +478,8 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
         hipLaunchKernelGGL((mhffn_bwd_dkdudv_kernel<DH>), grid, dim3(256), smem, st, a);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
+    }
+    if (phases & 8) {
         const long wsz = (long)d.Hkuv * d.E * d.d_e * d.d_h;
         const unsigned rblocks = (unsigned)((wsz / 4 + 255) / 256);
         if (grad_w_f32)
@@ -490,12 +495,12 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
 
 hipError_t launch_bwd_bf16(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
                            void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32, void* ws, const Dims& d,
-                           hipStream_t st)
+                           hipStream_t st, int phases)
 {
     switch (d.d_h) {
-        case 64: return launch_bwd_t<64>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, d, st);
-        case 96: return launch_bwd_t<96>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, d, st);
-        case 128: return launch_bwd_t<128>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, d, st);
+        case 64: return launch_bwd_t<64>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, d, st, phases);
+        case 96: return launch_bwd_t<96>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, d, st, phases);
+        case 128: return launch_bwd_t<128>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, d, st, phases);
     }
     return hipErrorInvalidValue;
 }

@@ -63,8 +63,9 @@ size_t mhffn_bwd_workspace_bytes(const mhffn_dims* dims, int dtype)
     return mhffn::bwd_workspace_bytes_bf16(to_dims(dims));
 }
 
-int mhffn_fwd(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
-              void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream)
+int mhffn_fwd_phases(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
+                     void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream,
+                     int phases)
 {
     const int rc = check_dims_impl(dims, dtype);
     if (rc != MHFFN_OK) return rc;
@@ -74,13 +75,20 @@ int mhffn_fwd(const void* Q, const void* K, const void* U, const void* V, const 
         return MHFFN_ERR_ALIGNMENT;
     const mhffn::Dims d = to_dims(dims);
     if (!workspace || workspace_bytes < mhffn::fwd_workspace_bytes_bf16(d)) return MHFFN_ERR_WORKSPACE;
-    const hipError_t err = mhffn::launch_fwd_bf16(Q, K, U, V, R, O, workspace, d, (hipStream_t)stream);
+    const hipError_t err = mhffn::launch_fwd_bf16(Q, K, U, V, R, O, workspace, d, (hipStream_t)stream, phases);
     return err == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
 }
 
-int mhffn_bwd(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
-              void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_dtype,
+int mhffn_fwd(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
               void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream)
+{
+    return mhffn_fwd_phases(Q, K, U, V, R, O, workspace, workspace_bytes, dims, dtype, stream, MHFFN_FWD_ALL);
+}
+
+int mhffn_bwd_phases(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
+                     void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_dtype,
+                     void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream,
+                     int phases)
 {
     const int rc = check_dims_impl(dims, dtype);
     if (rc != MHFFN_OK) return rc;
@@ -92,8 +100,17 @@ int mhffn_bwd(const void* Q, const void* K, const void* U, const void* V, const 
     const mhffn::Dims d = to_dims(dims);
     if (!workspace || workspace_bytes < mhffn::bwd_workspace_bytes_bf16(d)) return MHFFN_ERR_WORKSPACE;
     const hipError_t err = mhffn::launch_bwd_bf16(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR,
-                                                  grad_w_dtype == MHFFN_DTYPE_F32, workspace, d, (hipStream_t)stream);
+                                                  grad_w_dtype == MHFFN_DTYPE_F32, workspace, d, (hipStream_t)stream,
+                                                  phases);
     return err == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
+}
+
+int mhffn_bwd(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
+              void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_dtype,
+              void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream)
+{
+    return mhffn_bwd_phases(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_dtype, workspace, workspace_bytes, dims,
+                            dtype, stream, MHFFN_BWD_ALL);
 }
 
 }  // extern "C"

@@ -82,9 +82,9 @@ size_t packed_weights_bytes(const Dims& d, int bundle);
 size_t fwd_workspace_bytes_bf16(const Dims& d);
 size_t bwd_workspace_bytes_bf16(const Dims& d);
 hipError_t launch_fwd_bf16(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
-                           void* ws, const Dims& d, hipStream_t st);
+                           void* ws, const Dims& d, hipStream_t st, int phases);
 hipError_t launch_bwd_bf16(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
                            void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32,
-                           void* ws, const Dims& d, hipStream_t st);
+                           void* ws, const Dims& d, hipStream_t st, int phases);
 
 }  // namespace mhffn

@@ -168,10 +168,13 @@ static hipError_t launch_fwd_t(const FwdArgs& a, const Dims& d, hipStream_t st)
 }
 
 hipError_t launch_fwd_bf16(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
-                           void* ws, const Dims& d, hipStream_t st)
+                           void* ws, const Dims& d, hipStream_t st, int phases)
 {
-    hipError_t err = launch_pack_weights(K, U, V, ws, 0, d, st);
-    if (err != hipSuccess) return err;
+    if (phases & 1) {
+        hipError_t err = launch_pack_weights(K, U, V, ws, 0, d, st);
+        if (err != hipSuccess) return err;
+    }
+    if (!(phases & 2)) return hipSuccess;
     FwdArgs a{(const bf16_t*)Q, (const bf16_t*)ws, R, (bf16_t*)O, d.H, d.H / d.Hkuv, d.S, d.E, d.d_e / JB};
     switch (d.d_h) {
         case 64: return launch_fwd_t<64, 2>(a, d, st);

@@ -90,6 +90,25 @@ int mhffn_bwd(const void* Q, const void* K, const void* U, const void* V, const 
               void* workspace, size_t workspace_bytes,
               const mhffn_dims* dims, int dtype, void* stream);
 
+/* Phase-selectable variants for profiling: run only the kernels whose bit is set in `phases`, on a workspace that an
+ * earlier full call with the same arguments has filled.  mhffn_fwd == mhffn_fwd_phases(..., MHFFN_FWD_ALL) and
+ * mhffn_bwd == mhffn_bwd_phases(..., MHFFN_BWD_ALL).  They exist so a benchmark can bracket one kernel with HIP
+ * events on the launch stream; the reference has no counterpart (its kernels are launched one per Python call,
+ * flash_mlp_moe.py:832-866). */
+enum {
+    MHFFN_FWD_PACK = 1, MHFFN_FWD_MAIN = 2, MHFFN_FWD_ALL = 3,
+    MHFFN_BWD_PACK = 1, MHFFN_BWD_DQDR = 2, MHFFN_BWD_DKDUDV = 4, MHFFN_BWD_REDUCE = 8, MHFFN_BWD_ALL = 15
+};
+int mhffn_fwd_phases(const void* Q, const void* K, const void* U, const void* V, const float* R,
+                     void* O, void* workspace, size_t workspace_bytes,
+                     const mhffn_dims* dims, int dtype, void* stream, int phases);
+int mhffn_bwd_phases(const void* Q, const void* K, const void* U, const void* V, const float* R,
+                     const void* dO,
+                     void* dQ, void* dK, void* dU, void* dV, float* dR,
+                     int grad_w_dtype,
+                     void* workspace, size_t workspace_bytes,
+                     const mhffn_dims* dims, int dtype, void* stream, int phases);
+
 #ifdef __cplusplus
 }
 #endif
