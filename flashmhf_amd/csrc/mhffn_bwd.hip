@@ -72,22 +72,22 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
 #pragma unroll
             for (int x = 0; x < 16; ++x) dq[i][ct][x] = 0.0f;
 
-    uint4 stg[NCH];
+    u32x4 stg[NCH];
     auto gload = [&](int blk) {
-        const uint4* src = reinterpret_cast<const uint4*>(img + (long)blk * STAGE);
-#pragma unroll
-        for (int i = 0; i < NCH; ++i) {
+        const u32x4* src = reinterpret_cast<const u32x4*>(img + (long)blk * STAGE);
+        static_for<NCH>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
             const int idx = tid + i * 256;
-            if (idx < CHUNKS) stg[i] = src[idx];
-        }
+            if (i * 256 + 255 < CHUNKS || idx < CHUNKS) stg[i] = src[idx];
+        });
     };
     auto lstore = [&](int st) {
-        uint4* dst = reinterpret_cast<uint4*>(lds + st * STAGE);
-#pragma unroll
-        for (int i = 0; i < NCH; ++i) {
+        u32x4* dst = reinterpret_cast<u32x4*>(lds + st * STAGE);
+        static_for<NCH>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
             const int idx = tid + i * 256;
-            if (idx < CHUNKS) dst[idx] = stg[i];
-        }
+            if (i * 256 + 255 < CHUNKS || idx < CHUNKS) dst[idx] = stg[i];
+        });
     };
 
     gload(0);
@@ -255,7 +255,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     const int ntile = p.G * p.B * nS;
     const int t_begin = (int)((long)ntile * z / p.nslice), t_end = (int)((long)ntile * (z + 1) / p.nslice);
 
-    uint4 sq[NQ], sg_[NQ];
+    u32x4 sq[NQ], sg_[NQ];
     float sr[3];   // up to 3 R elements per thread (32*E <= 768 -> E <= 24); larger E loops below
     auto tile_rowbase = [&](int tau, int& st) -> long {
         st = tau % nS;
@@ -273,11 +273,11 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
                 const int row = idx / (DH / 8), c8 = (idx % (DH / 8)) * 8;
                 const int t = st * 32 + row;
                 if (t < p.S) {
-                    sq[i] = *reinterpret_cast<const uint4*>(p.Q + (rb + t) * DH + c8);
-                    sg_[i] = *reinterpret_cast<const uint4*>(p.dO + (rb + t) * DH + c8);
+                    sq[i] = *reinterpret_cast<const u32x4*>(p.Q + (rb + t) * DH + c8);
+                    sg_[i] = *reinterpret_cast<const u32x4*>(p.dO + (rb + t) * DH + c8);
                 } else {
-                    sq[i] = make_uint4(0, 0, 0, 0);
-                    sg_[i] = make_uint4(0, 0, 0, 0);
+                    sq[i] = u32x4{0u, 0u, 0u, 0u};
+                    sg_[i] = u32x4{0u, 0u, 0u, 0u};
                 }
             }
         }
@@ -299,8 +299,8 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
             const int idx = tid + i * 256;
             if (idx < QCH) {
                 const int row = idx / (DH / 8), c8 = (idx % (DH / 8)) * 8;
-                *reinterpret_cast<uint4*>(sQ + row * Ge::NAT_LD + c8) = sq[i];
-                *reinterpret_cast<uint4*>(sG + row * Ge::NAT_LD + c8) = sg_[i];
+                *reinterpret_cast<u32x4*>(sQ + row * Ge::NAT_LD + c8) = sq[i];
+                *reinterpret_cast<u32x4*>(sG + row * Ge::NAT_LD + c8) = sg_[i];
             }
         }
 #pragma unroll

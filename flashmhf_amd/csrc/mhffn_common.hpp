@@ -17,6 +17,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace mhffn {
 
@@ -25,6 +26,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // 16-byte copy unit (native vector: stays in registers)
 
 constexpr int JB = 32;          // rows of K/U/V per block
 constexpr int PADE = 8;         // bf16 elements of padding per LDS row (16 bytes: rotates rows across banks)
@@ -56,6 +58,28 @@ struct Geo {
     static constexpr int FWD_STAGE = 2 * NAT_ELEMS + TR_ELEMS;       // Kn | Un | Vt
     static constexpr int DQ_STAGE = 3 * NAT_ELEMS + 2 * TR_ELEMS;    // Kn | Un | Vn | Kt | Ut
 };
+
+// Compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>).  Arrays indexed through it are
+// indexed by constants from the first optimisation pass on, so they are promoted to registers (never scratch).
+template <int I, int N>
+struct StaticFor {
+    template <class F>
+    __device__ __forceinline__ static void run(F&& f)
+    {
+        f(std::integral_constant<int, I>{});
+        StaticFor<I + 1, N>::run(f);
+    }
+};
+template <int N>
+struct StaticFor<N, N> {
+    template <class F>
+    __device__ __forceinline__ static void run(F&&) {}
+};
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    StaticFor<0, N>::run(f);
+}
 
 __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c)
 {

@@ -30,6 +30,8 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     constexpr int NCH = (CHUNKS + 255) / 256;         // chunks per thread
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     bf16_t* lds = reinterpret_cast<bf16_t*>(smem_raw);
+    constexpr int BT = 128 * NCT;                      // tokens per workgroup
+    float* sR = reinterpret_cast<float*>(smem_raw + 2 * STAGE * sizeof(bf16_t));   // [E][BT]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int h = blockIdx.x, tb = blockIdx.y, b = blockIdx.z;
@@ -60,37 +62,42 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
 #pragma unroll
             for (int x = 0; x < 16; ++x) oacc[i][ct][x] = 0.0f;
 
-    uint4 stg[NCH];
+    u32x4 stg[NCH];
     auto gload = [&](int blk) {
-        const uint4* src = reinterpret_cast<const uint4*>(img + (long)blk * STAGE);
-#pragma unroll
-        for (int i = 0; i < NCH; ++i) {
+        const u32x4* src = reinterpret_cast<const u32x4*>(img + (long)blk * STAGE);
+        static_for<NCH>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
             const int idx = tid + i * 256;
-            if (idx < CHUNKS) stg[i] = src[idx];
-        }
+            if (i * 256 + 255 < CHUNKS || idx < CHUNKS) stg[i] = src[idx];
+        });
     };
     auto lstore = [&](int st) {
-        uint4* dst = reinterpret_cast<uint4*>(lds + st * STAGE);
-#pragma unroll
-        for (int i = 0; i < NCH; ++i) {
+        u32x4* dst = reinterpret_cast<u32x4*>(lds + st * STAGE);
+        static_for<NCH>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
             const int idx = tid + i * 256;
-            if (idx < CHUNKS) dst[idx] = stg[i];
-        }
+            if (i * 256 + 255 < CHUNKS || idx < CHUNKS) dst[idx] = stg[i];
+        });
     };
 
     gload(0);
+    // gate values of this workgroup's tokens, [E][BT] in LDS (read once per expert; keeps the main loop free of
+    // global loads other than the stage prefetch)
+    for (int idx = tid; idx < BT * p.E; idx += 256) {
+        int t = tb * BT + idx / p.E;
+        t = t < p.S ? t : p.S - 1;
+        sR[(idx % p.E) * BT + idx / p.E] = p.R[(rowbase + t) * p.E + idx % p.E];
+    }
     lstore(0);
-    if (nblk > 1) gload(1);
+    __syncthreads();
 
     float r[NCT];
     int blk = 0;
     for (int e = 0; e < p.E; ++e) {
 #pragma unroll
-        for (int ct = 0; ct < NCT; ++ct) r[ct] = p.R[trow[ct] * p.E + e];
+        for (int ct = 0; ct < NCT; ++ct) r[ct] = sR[e * BT + wave * (32 * NCT) + ct * 32 + l32];
         for (int jb = 0; jb < p.nbe; ++jb, ++blk) {
-            __syncthreads();   // stage blk&1 is complete; every wave has finished reading stage (blk+1)&1
-            if (blk + 1 < nblk) lstore((blk + 1) & 1);
-            if (blk + 2 < nblk) gload(blk + 2);
+            if (blk + 1 < nblk) gload(blk + 1);
 
             const bf16_t* sK = lds + (blk & 1) * STAGE;
             const bf16_t* sU = sK + Ge::NAT_ELEMS;
@@ -133,6 +140,8 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
 #pragma unroll
                     for (int ct = 0; ct < NCT; ++ct) oacc[i][ct] = mfma32(av, pt[ct][s], oacc[i][ct]);
                 }
+            if (blk + 1 < nblk) lstore((blk + 1) & 1);   // the other stage: last read before the previous barrier
+            __syncthreads();
         }
     }
 
@@ -160,8 +169,16 @@ size_t fwd_workspace_bytes_bf16(const Dims& d) { return packed_weights_bytes(d, 
 template <int DH, int NCT>
 static hipError_t launch_fwd_t(const FwdArgs& a, const Dims& d, hipStream_t st)
 {
-    constexpr int smem = 2 * Geo<DH>::FWD_STAGE * (int)sizeof(bf16_t);
     const int tokw = 128 * NCT;
+    const int smem = 2 * Geo<DH>::FWD_STAGE * (int)sizeof(bf16_t) + d.E * tokw * (int)sizeof(float);
+    if (smem > 160 * 1024) return hipErrorInvalidValue;
+    static int attr_smem = 0;   // dynamic LDS above 64 KB must be opted into, per kernel
+    if (smem > 64 * 1024 && smem > attr_smem) {
+        hipError_t e = hipFuncSetAttribute((const void*)mhffn_fwd_kernel<DH, NCT>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return e;
+        attr_smem = smem;
+    }
     dim3 grid((unsigned)d.H, (unsigned)((d.S + tokw - 1) / tokw), (unsigned)d.B);   // head fastest: one head per XCD
     hipLaunchKernelGGL((mhffn_fwd_kernel<DH, NCT>), grid, dim3(256), smem, st, a);
     return hipGetLastError();
