@@ -217,16 +217,22 @@ __device__ __forceinline__ bf16x8 lds_read_tr8(const bf16_t* p0, const bf16_t* p
     return r;
 }
 
+// LDS tile layout used by this kernel: 32 token rows of 256 bytes (16 chunks of 8 bf16; d_h/8 of them used); the
+// chunk that holds columns [8c, 8c+8) of row r sits at chunk position c ^ swz16(r).  With this XOR swizzle both
+// access patterns of the kernel -- 16-byte row reads (lanes = 16 different rows) and transposing 8-byte reads
+// (4 rows x 32 contiguous bytes per 16-lane group) -- are free of bank conflicts without padding, which lets the
+// tiles be filled by global_load_lds_dwordx4 (LDS destination = base + lane * 16).
+__device__ __forceinline__ int swz16(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+
 template <int DH>
 __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
 {
-    using Ge = Geo<DH>;
     constexpr int KS = DH / 16, CT = DH / 32;
-    constexpr int RLD = 36;                           // floats per expert row of the staged R tile (32 + 4 pad)
-    constexpr int QCH = JB * DH / 8;                  // 16-byte chunks of one Q (or dO) tile
-    constexpr int NQ = (QCH + 255) / 256;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    const int stage_bytes = 2 * Ge::NAT_ELEMS * 2 + p.E * RLD * 4;
+    constexpr int NCHUNK = DH / 8;                    // 16-byte chunks per token row
+    constexpr int TILE_B = JB * 256;                  // bytes of one staged Q (or dO) tile
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+    const int e_pad = (p.E + 1) & ~1;
+    const int stage_bytes = 2 * TILE_B + e_pad * 128;  // Q tile | dO tile | R tile [E][32] fp32
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int hk = blockIdx.y, z = blockIdx.z;
@@ -255,84 +261,60 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     const int ntile = p.G * p.B * nS;
     const int t_begin = (int)((long)ntile * z / p.nslice), t_end = (int)((long)ntile * (z + 1) / p.nslice);
 
-    u32x4 sq[NQ], sg_[NQ];
-    float sr[3];   // up to 3 R elements per thread (32*E <= 768 -> E <= 24); larger E loops below
-    auto tile_rowbase = [&](int tau, int& st) -> long {
-        st = tau % nS;
+    typedef const __attribute__((address_space(1))) void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    // Asynchronous fill of one stage: every wave issues its share of LDS-direct loads (no staging registers).
+    auto issue_tile = [&](int tau, int sidx) {
+        const int st = tau % nS;
         const int bb = (tau / nS) % p.B;
         const int gi = tau / (nS * p.B);
-        return ((long)bb * p.H + hk * p.G + gi) * p.S;
-    };
-    auto gload = [&](int tau) {
-        int st;
-        const long rb = tile_rowbase(tau, st);
+        const long rb = ((long)bb * p.H + hk * p.G + gi) * p.S;
+        unsigned char* sbase = smem_raw + sidx * stage_bytes;
+        // Q and dO: 8 wave-instructions each (4 rows of 256 B per instruction); wave w takes instructions w and w+4.
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) {
-            const int idx = tid + i * 256;
-            if (idx < QCH) {
-                const int row = idx / (DH / 8), c8 = (idx % (DH / 8)) * 8;
-                const int t = st * 32 + row;
-                if (t < p.S) {
-                    sq[i] = *reinterpret_cast<const u32x4*>(p.Q + (rb + t) * DH + c8);
-                    sg_[i] = *reinterpret_cast<const u32x4*>(p.dO + (rb + t) * DH + c8);
-                } else {
-                    sq[i] = u32x4{0u, 0u, 0u, 0u};
-                    sg_[i] = u32x4{0u, 0u, 0u, 0u};
-                }
-            }
+        for (int k = 0; k < 2; ++k) {
+            const int ins = wave + 4 * k;
+            const int r = 4 * ins + (lane >> 4);
+            int c = (lane & 15) ^ swz16(r);
+            c = c < NCHUNK ? c : 0;                   // unused chunk positions of narrow rows load a dummy chunk
+            int t = st * 32 + r;
+            t = t < p.S ? t : p.S - 1;                // tail rows are neutralised by r = 0 below
+            const long off = (rb + t) * DH + c * 8;
+            __builtin_amdgcn_global_load_lds((gptr_t)(p.Q + off), (lptr_t)(sbase + ins * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(p.dO + off), (lptr_t)(sbase + TILE_B + ins * 1024), 16, 0, 0);
         }
-#pragma unroll
-        for (int i = 0; i < 3; ++i) {
-            const int idx = tid + i * 256;
-            if (idx < 32 * p.E) {
-                const int t = st * 32 + idx / p.E;
-                sr[i] = t < p.S ? p.R[(rb + t) * p.E + idx % p.E] : 0.0f;
-            }
-        }
-    };
-    auto lstore = [&](int sidx) {
-        bf16_t* sQ = reinterpret_cast<bf16_t*>(smem_raw + sidx * stage_bytes);
-        bf16_t* sG = sQ + Ge::NAT_ELEMS;
-        float* sR = reinterpret_cast<float*>(sG + Ge::NAT_ELEMS);
-#pragma unroll
-        for (int i = 0; i < NQ; ++i) {
-            const int idx = tid + i * 256;
-            if (idx < QCH) {
-                const int row = idx / (DH / 8), c8 = (idx % (DH / 8)) * 8;
-                *reinterpret_cast<u32x4*>(sQ + row * Ge::NAT_LD + c8) = sq[i];
-                *reinterpret_cast<u32x4*>(sG + row * Ge::NAT_LD + c8) = sg_[i];
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < 3; ++i) {
-            const int idx = tid + i * 256;
-            if (idx < 32 * p.E) sR[(idx % p.E) * RLD + idx / p.E] = sr[i];
+        // R tile: [E][32] fp32, one 4-byte element per lane, two experts per instruction.
+        for (int ins = wave; 2 * ins < p.E; ins += 4) {
+            int e = 2 * ins + (lane >> 5);
+            e = e < p.E ? e : p.E - 1;
+            int t = st * 32 + l32;
+            t = t < p.S ? t : p.S - 1;
+            __builtin_amdgcn_global_load_lds((gptr_t)(p.R + (rb + t) * p.E + e),
+                                             (lptr_t)(sbase + 2 * TILE_B + ins * 256), 4, 0, 0);
         }
     };
 
-    if (t_begin < t_end) {
-        gload(t_begin);
-        lstore(0);
-        if (t_begin + 1 < t_end) gload(t_begin + 1);
-    }
+    if (t_begin < t_end) issue_tile(t_begin, 0);
 
+    const int lam = lane & 15;
     for (int tau = t_begin; tau < t_end; ++tau) {
         const int cur = (tau - t_begin) & 1;
-        __syncthreads();
-        if (tau + 1 < t_end) lstore(cur ^ 1);
-        if (tau + 2 < t_end) gload(tau + 2);
-        if (!active) continue;   // uniform per wave; idle waves still stage tiles and meet the barrier above
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's share of stage `cur` has landed
+        __syncthreads();                      // ... and everybody's; all waves are done reading the other stage
+        if (tau + 1 < t_end) issue_tile(tau + 1, cur ^ 1);
+        // waves beyond the last block recompute block nblk-1 (straight-line code) and drop their result at the end
 
-        const bf16_t* sQ = reinterpret_cast<const bf16_t*>(smem_raw + cur * stage_bytes);
-        const bf16_t* sG = sQ + Ge::NAT_ELEMS;
-        const float* sR = reinterpret_cast<const float*>(sG + Ge::NAT_ELEMS) + e_w * RLD;
+        const unsigned char* sQ = smem_raw + cur * stage_bytes;
+        const unsigned char* sG = sQ + TILE_B;
+        const float* sR = reinterpret_cast<const float*>(sG + TILE_B) + e_w * 32;
 
         f32x16 m, n, da;
 #pragma unroll
         for (int x = 0; x < 16; ++x) { m[x] = 0.0f; n[x] = 0.0f; da[x] = 0.0f; }
+        const int fr = swz16(l32);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const int off = l32 * Ge::NAT_LD + ks * 16 + 8 * g;
+            const int off = l32 * 256 + (((2 * ks + g) ^ fr) << 4);
             const bf16x8 aq = *reinterpret_cast<const bf16x8*>(sQ + off);
             const bf16x8 ag = *reinterpret_cast<const bf16x8*>(sG + off);
             m = mfma32(aq, kB[ks], m);
@@ -341,10 +323,13 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         }
 
         // registers 4a+b of m/n/da are token 8a + 4g + b (rows), column j = l32.
+        const int nvalid = p.S - (tau % nS) * 32;     // tokens of this tile that exist (>= 32 except in a tail tile)
         bf16x8 pB[2], dmB[2], dnB[2];
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
-            const f32x4 rv = *reinterpret_cast<const f32x4*>(sR + 8 * a + 4 * g);
+            f32x4 rv = *reinterpret_cast<const f32x4*>(sR + 8 * a + 4 * g);
+#pragma unroll
+            for (int bb = 0; bb < 4; ++bb) rv[bb] = (8 * a + 4 * g + bb < nvalid) ? rv[bb] : 0.0f;
 #pragma unroll
             for (int bb = 0; bb < 4; ++bb) {
                 const int i = 4 * a + bb;
@@ -357,19 +342,23 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
                 dnB[i >> 3][i & 7] = (bf16_t)(ra * sl);
                 dmB[i >> 3][i & 7] = (bf16_t)(ra * (nn * w));
             }
+            __builtin_amdgcn_sched_barrier(0);   // bound the number of element chains in flight (register pressure)
         }
 
-        // token contraction: A = Q^T / dO^T gathered from the natural tiles with transposing LDS reads.
-        // k-slot (s, g, kk) of the B operands is token 16s + 8(kk/4) + 4g + kk%4.
-        const int lam = lane & 15, chalf = (l32 >> 4) * 16;
+        // token contraction: A = Q^T / dO^T gathered from the row-major tiles with transposing LDS reads.
+        // k-slot (s, g, kk) of the B operands is token 16s + 8(kk/4) + 4g + kk%4; a 16-lane group covers 16 columns c.
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                const int col = 32 * ct + chalf + 4 * (lam & 3);
                 const int row0 = 16 * s + 4 * g + (lam >> 2);
-                const bf16x8 aqt = lds_read_tr8(sQ + row0 * Ge::NAT_LD + col, sQ + (row0 + 8) * Ge::NAT_LD + col);
-                const bf16x8 agt = lds_read_tr8(sG + row0 * Ge::NAT_LD + col, sG + (row0 + 8) * Ge::NAT_LD + col);
+                const int chunk = 4 * ct + 2 * (l32 >> 4) + ((lam & 3) >> 1);
+                const int o0 = row0 * 256 + ((chunk ^ swz16(row0)) << 4) + (lam & 1) * 8;
+                const int o1 = (row0 + 8) * 256 + ((chunk ^ swz16(row0 + 8)) << 4) + (lam & 1) * 8;
+                const bf16x8 aqt = lds_read_tr8(reinterpret_cast<const bf16_t*>(sQ + o0),
+                                                reinterpret_cast<const bf16_t*>(sQ + o1));
+                const bf16x8 agt = lds_read_tr8(reinterpret_cast<const bf16_t*>(sG + o0),
+                                                reinterpret_cast<const bf16_t*>(sG + o1));
                 dk[ct] = mfma32(aqt, dmB[s], dk[ct]);
                 du[ct] = mfma32(aqt, dnB[s], du[ct]);
                 dv[ct] = mfma32(agt, pB[s], dv[ct]);
@@ -471,7 +460,7 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
     if (phases & 4) {
         DwArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, part,
                  d.B, d.H, G, d.S, d.E, nbe, nslice};
-        const int smem = 2 * (2 * Geo<DH>::NAT_ELEMS * 2 + d.E * 36 * 4);
+        const int smem = 2 * (2 * JB * 256 + ((d.E + 1) & ~1) * 128);
         if (smem > 64 * 1024) return hipErrorInvalidValue;
         const int nblk = d.E * nbe;
         dim3 grid((unsigned)((nblk + 3) / 4), (unsigned)d.Hkuv, (unsigned)nslice);
