@@ -203,8 +203,6 @@ struct DwArgs {
     int B, H, G, S, E, nbe, nslice;
 };
 
-typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 v4bf16_t;
-
 __device__ __forceinline__ bf16x8 lds_read_tr8(const bf16_t* p0, const bf16_t* p1)
 {
     // Each call returns, for this lane's column, 4 + 4 consecutive rows of a row-major LDS tile (see the kernel).
@@ -217,20 +215,12 @@ __device__ __forceinline__ bf16x8 lds_read_tr8(const bf16_t* p0, const bf16_t* p
     return r;
 }
 
-// LDS tile layout used by this kernel: 32 token rows of 256 bytes (16 chunks of 8 bf16; d_h/8 of them used); the
-// chunk that holds columns [8c, 8c+8) of row r sits at chunk position c ^ swz16(r).  With this XOR swizzle both
-// access patterns of the kernel -- 16-byte row reads (lanes = 16 different rows) and transposing 8-byte reads
-// (4 rows x 32 contiguous bytes per 16-lane group) -- are free of bank conflicts without padding, which lets the
-// tiles be filled by global_load_lds_dwordx4 (LDS destination = base + lane * 16).
-__device__ __forceinline__ int swz16(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
-
 template <int DH>
 __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
 {
     constexpr int KS = DH / 16, CT = DH / 32;
     constexpr int NCHUNK = DH / 8;                    // 16-byte chunks per token row
-    constexpr int TILE_B = JB * 256;                  // bytes of one staged Q (or dO) tile
-    extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+        extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
     const int e_pad = (p.E + 1) & ~1;
     const int stage_bytes = 2 * TILE_B + e_pad * 128;  // Q tile | dO tile | R tile [E][32] fp32
 
@@ -261,8 +251,6 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     const int ntile = p.G * p.B * nS;
     const int t_begin = (int)((long)ntile * z / p.nslice), t_end = (int)((long)ntile * (z + 1) / p.nslice);
 
-    typedef const __attribute__((address_space(1))) void* gptr_t;
-    typedef __attribute__((address_space(3))) void* lptr_t;
     // Asynchronous fill of one stage: every wave issues its share of LDS-direct loads (no staging registers).
     auto issue_tile = [&](int tau, int sidx) {
         const int st = tau % nS;

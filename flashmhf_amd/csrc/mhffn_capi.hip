@@ -74,7 +74,8 @@ int mhffn_fwd_phases(const void* Q, const void* K, const void* U, const void* V,
         !aligned16(workspace))
         return MHFFN_ERR_ALIGNMENT;
     const mhffn::Dims d = to_dims(dims);
-    if (!workspace || workspace_bytes < mhffn::fwd_workspace_bytes_bf16(d)) return MHFFN_ERR_WORKSPACE;
+    const size_t need = mhffn::fwd_workspace_bytes_bf16(d);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return MHFFN_ERR_WORKSPACE;
     const hipError_t err = mhffn::launch_fwd_bf16(Q, K, U, V, R, O, workspace, d, (hipStream_t)stream, phases);
     return err == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
 }
@@ -98,7 +99,8 @@ int mhffn_bwd_phases(const void* Q, const void* K, const void* U, const void* V,
     for (const void* p : ptrs)
         if (!aligned16(p)) return MHFFN_ERR_ALIGNMENT;
     const mhffn::Dims d = to_dims(dims);
-    if (!workspace || workspace_bytes < mhffn::bwd_workspace_bytes_bf16(d)) return MHFFN_ERR_WORKSPACE;
+    const size_t need = mhffn::bwd_workspace_bytes_bf16(d);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return MHFFN_ERR_WORKSPACE;
     const hipError_t err = mhffn::launch_bwd_bf16(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR,
                                                   grad_w_dtype == MHFFN_DTYPE_F32, workspace, d, (hipStream_t)stream,
                                                   phases);

@@ -92,6 +92,67 @@ __device__ __forceinline__ float fast_sigmoid(float x)
     return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-LOG2E * x));
 }
 
+// ---- LDS tile layout shared by the main kernels -------------------------------------------------------------------
+// A staged tile is 32 rows (weight rows j, or tokens) of 256 bytes: 16 chunks of 8 bf16, d_h/8 of them used.  The chunk
+// holding columns [8c, 8c+8) of row r sits at chunk position c ^ swz16(r).  With this XOR swizzle both access patterns
+// -- 16-byte row reads (16 lanes = 16 different rows, same column chunk) and transposing 8-byte reads (a 16-lane group
+// reads 4 consecutive rows x 32 contiguous bytes) -- are bank-conflict free without padding, so tiles can be filled
+// by global_load_lds_dwordx4, whose LDS destination is (wave-uniform base) + lane * 16.
+constexpr int TILE_ROW_B = 256;
+constexpr int TILE_B = JB * TILE_ROW_B;   // 8 KB
+
+__device__ __forceinline__ int swz16(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 v4bf16_t;
+
+// One wave-instruction of an asynchronous tile fill: 4 rows (ins*4 .. ins*4+3) of a row-major [32][DH] bf16 source
+// tile whose row `r` starts at src_row0 + r * row_stride (elements).  Counts as one vmcnt event.
+template <int DH>
+__device__ __forceinline__ void tile_fill_ins(const bf16_t* src_row0, long row_stride, unsigned char* lds_tile, int ins,
+                                              int lane)
+{
+    const int r = 4 * ins + (lane >> 4);
+    int c = (lane & 15) ^ swz16(r);
+    c = c < DH / 8 ? c : 0;   // chunk positions a narrow row does not use receive a dummy chunk
+    __builtin_amdgcn_global_load_lds((gptr_t)(src_row0 + r * row_stride + c * 8), (lptr_t)(lds_tile + ins * 1024), 16, 0,
+                                     0);
+}
+
+// A operand (32 rows x 16 k) for k-step ks from a swizzled tile, row-major use: lane holds row `row`, columns
+// 16ks + 8g .. +7.
+__device__ __forceinline__ bf16x8 tile_read_rows(const unsigned char* tile, int row, int ks, int g)
+{
+    return *reinterpret_cast<const bf16x8*>(tile + row * TILE_ROW_B + (((2 * ks + g) ^ swz16(row)) << 4));
+}
+
+// A operand (32 rows = tile columns 32ct + l32, 16 k = tile rows) from a swizzled tile, transposed use:
+// lane holds column 32ct + l32; its 8 k values are tile rows rlo + {0..3} then rhi + {0..3}.  rlo/rhi must be uniform
+// within each 16-lane group (they may depend on lane / 32).
+__device__ __forceinline__ bf16x8 tile_read_cols(const unsigned char* tile, int ct, int rlo, int rhi, int lane)
+{
+    typedef __attribute__((address_space(3))) v4bf16_t* lds_v4_ptr;
+    const int lam = lane & 15, l32 = lane & 31;
+    const int chunk = 4 * ct + 2 * (l32 >> 4) + ((lam & 3) >> 1);
+    const int r0 = rlo + (lam >> 2), r1 = rhi + (lam >> 2);
+    const unsigned char* p0 = tile + r0 * TILE_ROW_B + ((chunk ^ swz16(r0)) << 4) + (lam & 1) * 8;
+    const unsigned char* p1 = tile + r1 * TILE_ROW_B + ((chunk ^ swz16(r1)) << 4) + (lam & 1) * 8;
+    v4bf16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4_ptr)(p0));
+    v4bf16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4_ptr)(p1));
+    bf16x8 r;
+    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+    return r;
+}
+
+// s_waitcnt vmcnt(N) only (gfx9 encoding: vmcnt[3:0] at bits 3:0, vmcnt[5:4] at bits 15:14; other counters unconstrained).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
 // Host-side launch entry points (defined in the per-kernel .hip files).
 struct Dims {
     int B, H, Hkuv, S, d_h, E, d_e;

@@ -57,7 +57,7 @@ def test_check_dims_codes(L, dims, dtype, code):
     if code != 0:
         assert L.mhffn_fwd_workspace_bytes(d, dtype) == 0 and L.mhffn_bwd_workspace_bytes(d, dtype) == 0
     else:
-        assert L.mhffn_fwd_workspace_bytes(d, dtype) > 0 and L.mhffn_bwd_workspace_bytes(d, dtype) > 0
+        assert L.mhffn_bwd_workspace_bytes(d, dtype) > 0     # token-slice partials of dK/dU/dV
 
 
 def test_entry_points_validate_before_touching_the_gpu(L):
@@ -68,7 +68,7 @@ def test_entry_points_validate_before_touching_the_gpu(L):
     odd = ctypes.c_void_p(0x1008)
     ok = ctypes.c_void_p(0x1000)
     assert L.mhffn_fwd(odd, ok, ok, ok, ok, ok, ok, 1 << 30, d, 0, null) == _capi.ERR_ALIGNMENT
-    assert L.mhffn_fwd(ok, ok, ok, ok, ok, ok, ok, 16, d, 0, null) == _capi.ERR_WORKSPACE
+    assert L.mhffn_bwd(*([ok] * 11), 0, ok, 16, d, 0, null) == _capi.ERR_WORKSPACE
     assert L.mhffn_bwd(*([ok] * 11), 5, ok, 1 << 30, d, 0, null) == _capi.ERR_DTYPE
     bad = _capi.Dims(1, 2, 2, 64, 128, 2, 65)
     assert L.mhffn_fwd(ok, ok, ok, ok, ok, ok, ok, 1 << 30, bad, 0, null) == _capi.ERR_EXPERT_DIM
