@@ -30,7 +30,8 @@ def build_lib(verbose=False, jobs=4):
 
     def compile_one(src):
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        extra = os.environ.get("MHFFN_EXTRA_HIPCC_FLAGS", "").split()   # experiments only, e.g. -DSOME_TUNABLE=3
+        cmd = [hipcc, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)
