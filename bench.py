@@ -6,7 +6,7 @@
 One "step" = one forward + one backward of the fused operator (through the C ABI, on torch's current stream) over
 one synthetic batch already resident in HBM.  Prints ONE JSON line.  Credited FLOPs: F1 = 2*T*H*E*d_e*d_h per
 GEMM; forward 3*F1, backward 8*F1 (recompute M,N + dA + 2 dQ + dK + dU + dV), fwd+bwd 11*F1 -- recomputation beyond
-that (the two-kernel backward runs 11*F1 on the hardware) is not credited.
+that (the two-kernel backward runs 11*F1 on the hardware, 14*F1 with the forward) is not credited.
 """
 import argparse
 import json
@@ -70,7 +70,7 @@ def kernel_timings(w, ins, n=10):
     O, dQ = torch.empty_like(Q), torch.empty_like(Q)
     dK, dU, dV = (torch.empty_like(K) for _ in range(3))
     dR = torch.empty_like(R)
-    wsf = torch.empty(L.mhffn_fwd_workspace_bytes(dims, 0), dtype=torch.uint8, device=Q.device)
+    wsf = torch.empty(max(16, L.mhffn_fwd_workspace_bytes(dims, 0)), dtype=torch.uint8, device=Q.device)
     wsb = torch.empty(L.mhffn_bwd_workspace_bytes(dims, 0), dtype=torch.uint8, device=Q.device)
     st = torch.cuda.current_stream().cuda_stream
 
@@ -86,10 +86,9 @@ def kernel_timings(w, ins, n=10):
         assert rc == 0, rc
 
     fwd(_capi.FWD_ALL)
-    out = {"fwd_pack": time_events(lambda: fwd(_capi.FWD_PACK), n), "fwd_main": time_events(lambda: fwd(_capi.FWD_MAIN), n)}
+    out = {"fwd_main": time_events(lambda: fwd(_capi.FWD_MAIN), n)}
     if "bwd" in w["passes"]:
         bwd(_capi.BWD_ALL)
-        out["bwd_pack"] = time_events(lambda: bwd(_capi.BWD_PACK), n)
         out["bwd_dqdr"] = time_events(lambda: bwd(_capi.BWD_DQDR), n)
         out["bwd_dkdudv"] = time_events(lambda: bwd(_capi.BWD_DKDUDV), n)
         out["bwd_reduce"] = time_events(lambda: bwd(_capi.BWD_REDUCE), n)

@@ -22,46 +22,69 @@ namespace mhffn {
 struct DqArgs {
     const bf16_t* Q;
     const bf16_t* dO;
-    const bf16_t* W;   // packed stage images [Hkuv][E * d_e/32][DQ_STAGE]
+    const bf16_t* K;
+    const bf16_t* U;
+    const bf16_t* V;
     const float* R;
     bf16_t* dQ;
     float* dR;
     int H, G, S, E, nbe;
 };
 
+constexpr int DQ_NST = 4;                  // LDS stages (K | U | V tiles each)
+constexpr int DQ_STAGE_B = 3 * TILE_B;
+
 template <int DH, int NCT>
 __global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
 {
-    using Ge = Geo<DH>;
     constexpr int KS = DH / 16, CT = DH / 32;
-    constexpr int STAGE = Ge::DQ_STAGE;
-    constexpr int CHUNKS = STAGE / 8;
-    constexpr int NCH = (CHUNKS + 255) / 256;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    bf16_t* lds = reinterpret_cast<bf16_t*>(smem_raw);
+    constexpr int BT = 128 * NCT;
+    constexpr int FILL = 6;                // tile-fill wave-instructions per wave and block (3 tiles x 8 / 4 waves)
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    float* sR = reinterpret_cast<float*>(smem + DQ_NST * DQ_STAGE_B);   // [E][BT]
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int h = blockIdx.x, tb = blockIdx.y, b = blockIdx.z;
     const int hk = h / p.G;
     const long rowbase = ((long)b * p.H + h) * p.S;
-    const int tok0 = tb * (128 * NCT) + wave * (32 * NCT);
+    const int tok0 = tb * BT + wave * (32 * NCT);
     const int nblk = p.E * p.nbe;
-    const bf16_t* img = p.W + (long)hk * nblk * STAGE;
+    const bf16_t* Kh = p.K + (long)hk * nblk * JB * DH;
+    const long offU = p.U - p.K, offV = p.V - p.K;
+
+    auto issue_block = [&](int blk) {
+        const int bc = blk < nblk ? blk : nblk - 1;
+        unsigned char* st = smem + (blk % DQ_NST) * DQ_STAGE_B;
+        const long roff = (long)bc * JB * DH;
+#pragma unroll
+        for (int k = 0; k < FILL; ++k) {
+            const int id = wave + 4 * k;             // 0..23: tile id/8 (K, U, V), 4-row group id%8
+            const int which = id >> 3;
+            const long toff = which == 0 ? 0 : (which == 1 ? offU : offV);
+            tile_fill_ins<DH>(Kh + toff + roff, DH, st + which * TILE_B, id & 7, lane);
+        }
+    };
+    issue_block(0);
+    issue_block(1);
 
     bf16x8 q[NCT][KS], go[NCT][KS];
-    long trow[NCT];
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) {
         int t = tok0 + ct * 32 + l32;
         t = t < p.S ? t : p.S - 1;
-        trow[ct] = rowbase + t;
-        const bf16_t* qr = p.Q + trow[ct] * DH + 8 * g;
-        const bf16_t* gr = p.dO + trow[ct] * DH + 8 * g;
+        const bf16_t* qr = p.Q + (rowbase + t) * DH + 8 * g;
+        const bf16_t* gr = p.dO + (rowbase + t) * DH + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             q[ct][ks] = *reinterpret_cast<const bf16x8*>(qr + ks * 16);
             go[ct][ks] = *reinterpret_cast<const bf16x8*>(gr + ks * 16);
         }
+    }
+    for (int idx = tid; idx < BT * p.E; idx += 256) {
+        int t = tb * BT + idx / p.E;
+        t = t < p.S ? t : p.S - 1;
+        sR[(idx % p.E) * BT + idx / p.E] = p.R[(rowbase + t) * p.E + idx % p.E];
     }
 
     f32x16 dq[CT][NCT];
@@ -72,46 +95,23 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
 #pragma unroll
             for (int x = 0; x < 16; ++x) dq[i][ct][x] = 0.0f;
 
-    u32x4 stg[NCH];
-    auto gload = [&](int blk) {
-        const u32x4* src = reinterpret_cast<const u32x4*>(img + (long)blk * STAGE);
-        static_for<NCH>([&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            const int idx = tid + i * 256;
-            if (i * 256 + 255 < CHUNKS || idx < CHUNKS) stg[i] = src[idx];
-        });
-    };
-    auto lstore = [&](int st) {
-        u32x4* dst = reinterpret_cast<u32x4*>(lds + st * STAGE);
-        static_for<NCH>([&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            const int idx = tid + i * 256;
-            if (i * 256 + 255 < CHUNKS || idx < CHUNKS) dst[idx] = stg[i];
-        });
-    };
-
-    gload(0);
-    lstore(0);
-    if (nblk > 1) gload(1);
-
+    const int krow = row_perm32(l32);
     int blk = 0;
     for (int e = 0; e < p.E; ++e) {
-        float r[NCT], dr[NCT];
+        float dr[NCT];
 #pragma unroll
-        for (int ct = 0; ct < NCT; ++ct) {
-            r[ct] = p.R[trow[ct] * p.E + e];
-            dr[ct] = 0.0f;
-        }
+        for (int ct = 0; ct < NCT; ++ct) dr[ct] = 0.0f;
         for (int jb = 0; jb < p.nbe; ++jb, ++blk) {
+            wait_vmcnt<FILL>();       // block blk has landed (block blk+1 may be in flight)
             __syncthreads();
-            if (blk + 1 < nblk) lstore((blk + 1) & 1);
-            if (blk + 2 < nblk) gload(blk + 2);
+            issue_block(blk + 2);
 
-            const bf16_t* sK = lds + (blk & 1) * STAGE;
-            const bf16_t* sU = sK + Ge::NAT_ELEMS;
-            const bf16_t* sV = sU + Ge::NAT_ELEMS;
-            const bf16_t* sKt = sV + Ge::NAT_ELEMS;
-            const bf16_t* sUt = sKt + Ge::TR_ELEMS;
+            const unsigned char* sK = smem + (blk % DQ_NST) * DQ_STAGE_B;
+            const unsigned char* sU = sK + TILE_B;
+            const unsigned char* sV = sU + TILE_B;
+            float r[NCT];
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct) r[ct] = sR[e * BT + wave * (32 * NCT) + ct * 32 + l32];
 
             f32x16 m[NCT], n[NCT], da[NCT];
 #pragma unroll
@@ -120,10 +120,9 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
                 for (int x = 0; x < 16; ++x) { m[ct][x] = 0.0f; n[ct][x] = 0.0f; da[ct][x] = 0.0f; }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const int off = l32 * Ge::NAT_LD + ks * 16 + 8 * g;
-                const bf16x8 ak = *reinterpret_cast<const bf16x8*>(sK + off);
-                const bf16x8 au = *reinterpret_cast<const bf16x8*>(sU + off);
-                const bf16x8 av = *reinterpret_cast<const bf16x8*>(sV + off);
+                const bf16x8 ak = tile_read_rows(sK, krow, ks, g);
+                const bf16x8 au = tile_read_rows(sU, krow, ks, g);
+                const bf16x8 av = tile_read_rows(sV, krow, ks, g);
 #pragma unroll
                 for (int ct = 0; ct < NCT; ++ct) {
                     m[ct] = mfma32(ak, q[ct][ks], m[ct]);
@@ -145,7 +144,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
                         const float sl = x * sg;                 // silu(m)
                         const float as = a * sl;
                         dr[ct] = __builtin_fmaf(as, nn, dr[ct]);
-                        const float w = sg + sl * (1.0f - sg);    // silu'(m)
+                        const float w = __builtin_fmaf(sl, 1.0f - sg, sg);    // silu'(m)
                         dnt[ct][s][kk] = (bf16_t)(r[ct] * as);
                         dmt[ct][s][kk] = (bf16_t)((r[ct] * a) * (nn * w));
                     }
@@ -154,9 +153,8 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
             for (int i = 0; i < CT; ++i)
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    const int off = (i * 32 + l32) * Ge::TR_LD + 16 * s + 8 * g;
-                    const bf16x8 akt = *reinterpret_cast<const bf16x8*>(sKt + off);
-                    const bf16x8 aut = *reinterpret_cast<const bf16x8*>(sUt + off);
+                    const bf16x8 akt = tile_read_cols(sK, i, 16 * s + 8 * g, 16 * s + 8 * g + 4, lane);
+                    const bf16x8 aut = tile_read_cols(sU, i, 16 * s + 8 * g, 16 * s + 8 * g + 4, lane);
 #pragma unroll
                     for (int ct = 0; ct < NCT; ++ct) {
                         dq[i][ct] = mfma32(akt, dmt[ct][s], dq[i][ct]);
@@ -172,6 +170,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
             if (g == 0 && t < p.S) p.dR[(rowbase + t) * p.E + e] = tot;
         }
     }
+    wait_vmcnt<0>();   // drain the phantom prefetches before the workgroup's LDS is released
 
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) {
@@ -203,33 +202,23 @@ struct DwArgs {
     int B, H, G, S, E, nbe, nslice;
 };
 
-__device__ __forceinline__ bf16x8 lds_read_tr8(const bf16_t* p0, const bf16_t* p1)
-{
-    // Each call returns, for this lane's column, 4 + 4 consecutive rows of a row-major LDS tile (see the kernel).
-    typedef __attribute__((address_space(3))) v4bf16_t* lds_v4_ptr;
-    v4bf16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4_ptr)(p0));
-    v4bf16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4_ptr)(p1));
-    bf16x8 r;
-    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
-    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
-    return r;
-}
+constexpr int DW_RTILE_B = 16 * 1024;                 // staged R tile: [E][32] fp32, E <= 128
+constexpr int DW_STAGE_B = 2 * TILE_B + DW_RTILE_B;    // Q tile | dO tile | R tile
 
 template <int DH>
 __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
 {
     constexpr int KS = DH / 16, CT = DH / 32;
     constexpr int NCHUNK = DH / 8;                    // 16-byte chunks per token row
-        extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
-    const int e_pad = (p.E + 1) & ~1;
-    const int stage_bytes = 2 * TILE_B + e_pad * 128;  // Q tile | dO tile | R tile [E][32] fp32
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hk = blockIdx.y, z = blockIdx.z;
     const int nblk = p.E * p.nbe;
     const int jblk = blockIdx.x * 4 + wave;
     const bool active = jblk < nblk;
-    const int jb_c = active ? jblk : nblk - 1;
+    const int jb_c = active ? jblk : nblk - 1;        // idle waves of the last column recompute the last block
     const int e_w = jb_c / p.nbe;
     const long wrow = ((long)hk * nblk + jb_c) * JB + l32;      // this lane's row of K/U/V (column j of the products)
 
@@ -251,23 +240,34 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     const int ntile = p.G * p.B * nS;
     const int t_begin = (int)((long)ntile * z / p.nslice), t_end = (int)((long)ntile * (z + 1) / p.nslice);
 
-    // Asynchronous fill of one stage: every wave issues its share of LDS-direct loads (no staging registers).
-    auto issue_tile = [&](int tau, int sidx) {
-        const int st = tau % nS;
-        const int bb = (tau / nS) % p.B;
-        const int gi = tau / (nS * p.B);
-        const long rb = ((long)bb * p.H + hk * p.G + gi) * p.S;
-        unsigned char* sbase = smem_raw + sidx * stage_bytes;
-        // Q and dO: 8 wave-instructions each (4 rows of 256 B per instruction); wave w takes instructions w and w+4.
+    // Tile cursor of the prefetcher: tile index -> (q-head of the group, batch, 32-token tile), advanced incrementally.
+    int pf_st = t_begin % nS, pf_bb = (t_begin / nS) % p.B, pf_gi = t_begin / (nS * p.B);
+
+    // per-lane constants of the tile fill: this wave's two 4-row groups, swizzled source chunk
+    int fill_row[2], fill_coff[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int ins = wave + 4 * k;
+        const int r = 4 * ins + (lane >> 4);
+        int c = (lane & 15) ^ swz16(r);
+        c = c < NCHUNK ? c : 0;                       // unused chunk positions of narrow rows load a dummy chunk
+        fill_row[k] = r;
+        fill_coff[k] = c * 8;
+    }
+
+    // Asynchronous fill of stage `sidx` with the tile under the cursor; every wave issues its share of LDS-direct
+    // loads (no staging registers), then the cursor advances.  Rows past the end of a sequence are clamped to its last
+    // row and their gate value is zeroed afterwards (zero_tail), which removes them from all three products.
+    auto issue_tile = [&](int sidx) {
+        const long rb = ((long)pf_bb * p.H + hk * p.G + pf_gi) * p.S;
+        const int t0 = pf_st * 32;
+        unsigned char* sbase = smem_raw + sidx * DW_STAGE_B;
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
+            int t = t0 + fill_row[k];
+            t = t < p.S ? t : p.S - 1;
+            const long off = (rb + t) * DH + fill_coff[k];
             const int ins = wave + 4 * k;
-            const int r = 4 * ins + (lane >> 4);
-            int c = (lane & 15) ^ swz16(r);
-            c = c < NCHUNK ? c : 0;                   // unused chunk positions of narrow rows load a dummy chunk
-            int t = st * 32 + r;
-            t = t < p.S ? t : p.S - 1;                // tail rows are neutralised by r = 0 below
-            const long off = (rb + t) * DH + c * 8;
             __builtin_amdgcn_global_load_lds((gptr_t)(p.Q + off), (lptr_t)(sbase + ins * 1024), 16, 0, 0);
             __builtin_amdgcn_global_load_lds((gptr_t)(p.dO + off), (lptr_t)(sbase + TILE_B + ins * 1024), 16, 0, 0);
         }
@@ -275,62 +275,73 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         for (int ins = wave; 2 * ins < p.E; ins += 4) {
             int e = 2 * ins + (lane >> 5);
             e = e < p.E ? e : p.E - 1;
-            int t = st * 32 + l32;
+            int t = t0 + l32;
             t = t < p.S ? t : p.S - 1;
             __builtin_amdgcn_global_load_lds((gptr_t)(p.R + (rb + t) * p.E + e),
                                              (lptr_t)(sbase + 2 * TILE_B + ins * 256), 4, 0, 0);
         }
+        if (++pf_st == nS) {
+            pf_st = 0;
+            if (++pf_bb == p.B) { pf_bb = 0; ++pf_gi; }
+        }
+    };
+    // Called by every wave after its own loads of stage `sidx` have landed and before the barrier that publishes
+    // the stage: zeroes the gate values of the rows a tail tile does not have.
+    auto zero_tail = [&](int sidx, int nvalid) {
+        float* sR = reinterpret_cast<float*>(smem_raw + sidx * DW_STAGE_B + 2 * TILE_B);
+        for (int ins = wave; 2 * ins < p.E; ins += 4)
+            if (l32 >= nvalid) sR[ins * 64 + lane] = 0.0f;
     };
 
-    if (t_begin < t_end) issue_tile(t_begin, 0);
+    int cur_st = pf_st;                                // 32-token tile index (within its sequence) of tile `tau`
+    if (t_begin < t_end) issue_tile(0);
 
-    const int lam = lane & 15;
-    for (int tau = t_begin; tau < t_end; ++tau) {
-        const int cur = (tau - t_begin) & 1;
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's share of stage `cur` has landed
+    const int fr = swz16(l32);
+    f32x16 zero16;
+#pragma unroll
+    for (int x = 0; x < 16; ++x) zero16[x] = 0.0f;
+
+    auto process = [&](auto stage_c, int tau) {
+        constexpr int cur = decltype(stage_c)::value;
+        wait_vmcnt<0>();                      // this wave's share of stage `cur` has landed
+        const int nvalid = p.S - cur_st * 32;
+        if (nvalid < 32) zero_tail(cur, nvalid);
+        if (++cur_st == nS) cur_st = 0;
         __syncthreads();                      // ... and everybody's; all waves are done reading the other stage
-        if (tau + 1 < t_end) issue_tile(tau + 1, cur ^ 1);
-        // waves beyond the last block recompute block nblk-1 (straight-line code) and drop their result at the end
+        if (tau + 1 < t_end) issue_tile(cur ^ 1);
 
-        const unsigned char* sQ = smem_raw + cur * stage_bytes;
+        const unsigned char* sQ = smem_raw + cur * DW_STAGE_B;
         const unsigned char* sG = sQ + TILE_B;
         const float* sR = reinterpret_cast<const float*>(sG + TILE_B) + e_w * 32;
 
         f32x16 m, n, da;
 #pragma unroll
-        for (int x = 0; x < 16; ++x) { m[x] = 0.0f; n[x] = 0.0f; da[x] = 0.0f; }
-        const int fr = swz16(l32);
-#pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const int off = l32 * 256 + (((2 * ks + g) ^ fr) << 4);
             const bf16x8 aq = *reinterpret_cast<const bf16x8*>(sQ + off);
             const bf16x8 ag = *reinterpret_cast<const bf16x8*>(sG + off);
-            m = mfma32(aq, kB[ks], m);
-            n = mfma32(aq, uB[ks], n);
-            da = mfma32(ag, vB[ks], da);
+            m = mfma32(aq, kB[ks], ks == 0 ? zero16 : m);
+            n = mfma32(aq, uB[ks], ks == 0 ? zero16 : n);
+            da = mfma32(ag, vB[ks], ks == 0 ? zero16 : da);
         }
 
         // registers 4a+b of m/n/da are token 8a + 4g + b (rows), column j = l32.
-        const int nvalid = p.S - (tau % nS) * 32;     // tokens of this tile that exist (>= 32 except in a tail tile)
         bf16x8 pB[2], dmB[2], dnB[2];
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
-            f32x4 rv = *reinterpret_cast<const f32x4*>(sR + 8 * a + 4 * g);
-#pragma unroll
-            for (int bb = 0; bb < 4; ++bb) rv[bb] = (8 * a + 4 * g + bb < nvalid) ? rv[bb] : 0.0f;
+            const f32x4 rv = *reinterpret_cast<const f32x4*>(sR + 8 * a + 4 * g);
 #pragma unroll
             for (int bb = 0; bb < 4; ++bb) {
                 const int i = 4 * a + bb;
                 const float x = m[i], nn = n[i], dA = da[i], rr = rv[bb];
                 const float sg = fast_sigmoid(x);
-                const float sl = x * sg;
-                const float w = sg + sl * (1.0f - sg);
-                const float ra = rr * dA;
-                pB[i >> 3][i & 7] = (bf16_t)(rr * (sl * nn));
-                dnB[i >> 3][i & 7] = (bf16_t)(ra * sl);
-                dmB[i >> 3][i & 7] = (bf16_t)(ra * (nn * w));
+                const float sl = x * sg;                               // silu(m)
+                const float w = __builtin_fmaf(sl, 1.0f - sg, sg);     // silu'(m)
+                const float rs = rr * sl;
+                pB[i >> 3][i & 7] = (bf16_t)(rs * nn);
+                dnB[i >> 3][i & 7] = (bf16_t)(rs * dA);
+                dmB[i >> 3][i & 7] = (bf16_t)((rr * w) * (nn * dA));
             }
-            __builtin_amdgcn_sched_barrier(0);   // bound the number of element chains in flight (register pressure)
         }
 
         // token contraction: A = Q^T / dO^T gathered from the row-major tiles with transposing LDS reads.
@@ -339,19 +350,21 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                const int row0 = 16 * s + 4 * g + (lam >> 2);
-                const int chunk = 4 * ct + 2 * (l32 >> 4) + ((lam & 3) >> 1);
-                const int o0 = row0 * 256 + ((chunk ^ swz16(row0)) << 4) + (lam & 1) * 8;
-                const int o1 = (row0 + 8) * 256 + ((chunk ^ swz16(row0 + 8)) << 4) + (lam & 1) * 8;
-                const bf16x8 aqt = lds_read_tr8(reinterpret_cast<const bf16_t*>(sQ + o0),
-                                                reinterpret_cast<const bf16_t*>(sQ + o1));
-                const bf16x8 agt = lds_read_tr8(reinterpret_cast<const bf16_t*>(sG + o0),
-                                                reinterpret_cast<const bf16_t*>(sG + o1));
+                const bf16x8 aqt = tile_read_cols(sQ, ct, 16 * s + 4 * g, 16 * s + 4 * g + 8, lane);
+                const bf16x8 agt = tile_read_cols(sG, ct, 16 * s + 4 * g, 16 * s + 4 * g + 8, lane);
                 dk[ct] = mfma32(aqt, dmB[s], dk[ct]);
                 du[ct] = mfma32(aqt, dnB[s], du[ct]);
                 dv[ct] = mfma32(agt, pB[s], dv[ct]);
             }
+    };
+
+    // two tiles per trip so that the LDS stage (and every LDS address) is a compile-time constant
+    int tau = t_begin;
+    for (; tau + 1 < t_end; tau += 2) {
+        process(std::integral_constant<int, 0>{}, tau);
+        process(std::integral_constant<int, 1>{}, tau + 1);
     }
+    if (tau < t_end) process(std::integral_constant<int, 0>{}, tau);
 
     if (active) {
         // dK^T registers 4a+b of row tile ct: c = 32ct + 8a + 4g + b, column j = l32 -> 16-byte runs along c.
@@ -411,7 +424,7 @@ static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 size_t bwd_workspace_bytes_bf16(const Dims& d)
 {
     const size_t wsz = (size_t)d.Hkuv * d.E * d.d_e * d.d_h;
-    return align256(packed_weights_bytes(d, 1)) + align256((size_t)pick_nslice(d) * 3 * wsz * sizeof(float));
+    return align256((size_t)pick_nslice(d) * 3 * wsz * sizeof(float));
 }
 
 template <int DH>
@@ -421,24 +434,22 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
 {
     constexpr int NCT = 2;
     hipError_t err = hipSuccess;
-    if (phases & 1) {
-        err = launch_pack_weights(K, U, V, ws, 1, d, st);
-        if (err != hipSuccess) return err;
-    }
-    float* part = reinterpret_cast<float*>((char*)ws + align256(packed_weights_bytes(d, 1)));
+    float* part = reinterpret_cast<float*>(ws);
     const int nbe = d.d_e / JB, G = d.H / d.Hkuv;
 
     if (phases & 2) {
-        DqArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)ws, R, (bf16_t*)dQ, dR, d.H, G, d.S, d.E, nbe};
-        constexpr int smem = 2 * Geo<DH>::DQ_STAGE * (int)sizeof(bf16_t);
-        static bool attr_done = false;   // raising the dynamic LDS limit is a per-process, per-kernel property
-        if (!attr_done) {
+        DqArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R,
+                 (bf16_t*)dQ, dR, d.H, G, d.S, d.E, nbe};
+        const int tokw = 128 * NCT;
+        const int smem = DQ_NST * DQ_STAGE_B + d.E * tokw * (int)sizeof(float);
+        if (smem > 160 * 1024) return hipErrorInvalidValue;
+        static int attr_smem = 0;   // dynamic LDS above 64 KB must be opted into, per kernel
+        if (smem > attr_smem) {
             err = hipFuncSetAttribute((const void*)mhffn_bwd_dqdr_kernel<DH, NCT>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
             if (err != hipSuccess) return err;
-            attr_done = true;
+            attr_smem = smem;
         }
-        const int tokw = 128 * NCT;
         dim3 grid((unsigned)d.H, (unsigned)((d.S + tokw - 1) / tokw), (unsigned)d.B);
         hipLaunchKernelGGL((mhffn_bwd_dqdr_kernel<DH, NCT>), grid, dim3(256), smem, st, a);
         err = hipGetLastError();
@@ -448,8 +459,8 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
     if (phases & 4) {
         DwArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, part,
                  d.B, d.H, G, d.S, d.E, nbe, nslice};
-        const int smem = 2 * (2 * JB * 256 + ((d.E + 1) & ~1) * 128);
-        if (smem > 64 * 1024) return hipErrorInvalidValue;
+        const int smem = 2 * DW_STAGE_B;
+        if (d.E > 128) return hipErrorInvalidValue;   // staged R tile holds at most 128 experts
         const int nblk = d.E * nbe;
         dim3 grid((unsigned)((nblk + 3) / 4), (unsigned)d.Hkuv, (unsigned)nslice);
         hipLaunchKernelGGL((mhffn_bwd_dkdudv_kernel<DH>), grid, dim3(256), smem, st, a);

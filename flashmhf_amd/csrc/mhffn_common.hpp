@@ -12,7 +12,7 @@
 //   through LDS: with the first product written "transposed" (rows = j, cols = t) registers 8s..8s+7 of lane
 //   (t, g = l/32) are exactly the 8 k-slots the second product's B operand wants, provided slot (s, g, kk)
 //   means j = 16s + 8g + kk.  That holds when output row rho of the first product was fed K row
-//   PI(rho) (see row_perm32): the permutation is applied once, when the weight tiles are packed.
+//   PI(rho) (see row_perm32): the permutation is applied in the LDS read address of the K/U/V tiles.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -29,7 +29,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // 16-byte copy unit (native vector: stays in registers)
 
 constexpr int JB = 32;          // rows of K/U/V per block
-constexpr int PADE = 8;         // bf16 elements of padding per LDS row (16 bytes: rotates rows across banks)
 constexpr float LOG2E = 1.4426950408889634f;
 
 // MFMA output row rho (0..31) -> which row of the 32-row weight block must be fed as A-row rho so that
@@ -45,19 +44,6 @@ __host__ __device__ constexpr int tok_perm32(int p)
 {
     return (p & 16) + 8 * ((p >> 2) & 1) + 4 * ((p >> 3) & 1) + (p & 3);
 }
-
-// Geometry of the packed tiles, all in bf16 elements.
-//   natural tile   [32 rows][DH + 8]   row rho = weight row row_perm32(rho) (or token row for Q/dO tiles)
-//   transposed tile [DH rows][32 + 8]  row c, position = j (weights) or tok_perm32 position (tokens)
-template <int DH>
-struct Geo {
-    static constexpr int NAT_LD = DH + PADE;
-    static constexpr int NAT_ELEMS = JB * NAT_LD;
-    static constexpr int TR_LD = JB + PADE;
-    static constexpr int TR_ELEMS = DH * TR_LD;
-    static constexpr int FWD_STAGE = 2 * NAT_ELEMS + TR_ELEMS;       // Kn | Un | Vt
-    static constexpr int DQ_STAGE = 3 * NAT_ELEMS + 2 * TR_ELEMS;    // Kn | Un | Vn | Kt | Ut
-};
 
 // Compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>).  Arrays indexed through it are
 // indexed by constants from the first optimisation pass on, so they are promoted to registers (never scratch).
@@ -157,12 +143,6 @@ __device__ __forceinline__ void wait_vmcnt()
 struct Dims {
     int B, H, Hkuv, S, d_h, E, d_e;
 };
-
-// Re-lays the K/U/V blocks of every (kuv-head, 32-row block) as one contiguous "stage image" that the main kernels
-// copy verbatim into LDS.  bundle 0: forward (Kn|Un|Vt); bundle 1: dQ/dR kernel (Kn|Un|Vn|Kt|Ut).
-hipError_t launch_pack_weights(const void* K, const void* U, const void* V, void* dst, int bundle, const Dims& d,
-                               hipStream_t st);
-size_t packed_weights_bytes(const Dims& d, int bundle);
 
 size_t fwd_workspace_bytes_bf16(const Dims& d);
 size_t bwd_workspace_bytes_bf16(const Dims& d);

@@ -91,7 +91,8 @@ int mhffn_bwd(const void* Q, const void* K, const void* U, const void* V, const 
               const mhffn_dims* dims, int dtype, void* stream);
 
 /* Phase-selectable variants for profiling: run only the kernels whose bit is set in `phases`, on a workspace that an
- * earlier full call with the same arguments has filled.  mhffn_fwd == mhffn_fwd_phases(..., MHFFN_FWD_ALL) and
+ * earlier full call with the same arguments has filled.  The *_PACK bits are accepted and do nothing (the kernels
+ * read K, U, V in place; there is no re-layout pass).  mhffn_fwd == mhffn_fwd_phases(..., MHFFN_FWD_ALL) and
  * mhffn_bwd == mhffn_bwd_phases(..., MHFFN_BWD_ALL).  They exist so a benchmark can bracket one kernel with HIP
  * events on the launch stream; the reference has no counterpart (its kernels are launched one per Python call,
  * flash_mlp_moe.py:832-866). */
