@@ -13,6 +13,7 @@ int check_dims_impl(const mhffn_dims* d, int dtype)
     if (d->B <= 0 || d->H <= 0 || d->Hkuv <= 0 || d->S <= 0 || d->E <= 0 || d->d_e <= 0 || d->d_h <= 0)
         return MHFFN_ERR_SHAPE;
     if (d->H % d->Hkuv != 0) return MHFFN_ERR_SHAPE;
+    if (d->E > 64) return MHFFN_ERR_SHAPE;   // the kernels stage a [E][256] fp32 gate tile in LDS next to the weight ring
     if (dtype == MHFFN_DTYPE_F32) return MHFFN_ERR_DTYPE;   // no fp32 kernels in this build
     if (d->d_h != 64 && d->d_h != 96 && d->d_h != 128) return MHFFN_ERR_HEAD_DIM;
     if (d->d_e % 32 != 0) return MHFFN_ERR_EXPERT_DIM;
@@ -35,7 +36,7 @@ const char* mhffn_strerror(int code)
         case MHFFN_ERR_DTYPE: return "unsupported dtype (Q, K, U, V must be bfloat16; R float32)";
         case MHFFN_ERR_HEAD_DIM: return "unsupported head dim (d_h must be 64, 96 or 128)";
         case MHFFN_ERR_EXPERT_DIM: return "unsupported expert dim (d_e must be a multiple of 32)";
-        case MHFFN_ERR_SHAPE: return "invalid extents (all must be positive, H a multiple of Hkuv)";
+        case MHFFN_ERR_SHAPE: return "invalid extents (all must be positive, H a multiple of Hkuv, E <= 64)";
         case MHFFN_ERR_WORKSPACE: return "workspace missing or too small";
         case MHFFN_ERR_LAUNCH: return "kernel launch failed";
         case MHFFN_ERR_ALIGNMENT: return "pointer not 16-byte aligned";

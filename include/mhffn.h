@@ -39,7 +39,7 @@ enum {
     MHFFN_ERR_DTYPE        = -2,  /* reference: TypeError, flash_mlp_moe.py:761-766; TORCH_CHECK flash_ffn_moe.cu:943-945 */
     MHFFN_ERR_HEAD_DIM     = -3,  /* reference: assert head_dim == 128, flash_ffn_moe.cu:956 */
     MHFFN_ERR_EXPERT_DIM   = -4,  /* reference: ValueError, flash_mlp_moe.py:758-759; assert flash_ffn_moe.cu:958 */
-    MHFFN_ERR_SHAPE        = -5,  /* non-positive extent, H not a multiple of Hkuv */
+    MHFFN_ERR_SHAPE        = -5,  /* non-positive extent, H not a multiple of Hkuv, E > 64 */
     MHFFN_ERR_WORKSPACE    = -6,  /* workspace missing or smaller than *_workspace_bytes() */
     MHFFN_ERR_LAUNCH       = -7,  /* hipGetLastError() after a launch */
     MHFFN_ERR_ALIGNMENT    = -8   /* a tensor or workspace pointer is not 16-byte aligned */
@@ -52,7 +52,7 @@ typedef struct mhffn_dims {
     int Hkuv;   /* K/U/V heads; H % Hkuv == 0 (grouped "GQ-FFN", flash_mlp_moe.py:194,222) */
     int S;      /* tokens per (batch, head) */
     int d_h;    /* head dim */
-    int E;      /* experts (sub-networks) per head */
+    int E;      /* experts (sub-networks) per head, at most 64 */
     int d_e;    /* rows of K/U/V per expert */
 } mhffn_dims;
 

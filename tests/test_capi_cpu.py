@@ -48,6 +48,7 @@ def test_strerror_and_is_supported(L):
     ((8, 8, 8, 2048, 100, 11, 352), 0, _capi.ERR_HEAD_DIM),
     ((8, 8, 3, 2048, 128, 11, 352), 0, _capi.ERR_SHAPE),
     ((0, 8, 8, 2048, 128, 11, 352), 0, _capi.ERR_SHAPE),
+    ((8, 8, 8, 2048, 128, 65, 352), 0, _capi.ERR_SHAPE),
     ((8, 8, 8, 2048, 128, 11, 352), 1, _capi.ERR_DTYPE),
     ((8, 8, 8, 2048, 128, 11, 352), 7, _capi.ERR_DTYPE),
 ])
