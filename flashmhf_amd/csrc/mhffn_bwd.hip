@@ -34,12 +34,13 @@ struct DqArgs {
 constexpr int DQ_NST = 4;                  // LDS stages (K | U | V tiles each)
 constexpr int DQ_STAGE_B = 3 * TILE_B;
 
-template <int DH, int NCT>
-__global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
+template <int DH, int NCT, int NW>
+__global__ __launch_bounds__(NW * 64) void mhffn_bwd_dqdr_kernel(DqArgs p)
 {
     constexpr int KS = DH / 16, CT = DH / 32;
-    constexpr int BT = 128 * NCT;
-    constexpr int FILL = 6;                // tile-fill wave-instructions per wave and block (3 tiles x 8 / 4 waves)
+    constexpr int BT = NW * 32 * NCT;
+    constexpr int NTHR = NW * 64;
+    constexpr int FILL = 24 / NW;          // tile-fill wave-instructions per wave and block (3 tiles x 8 / NW waves)
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     float* sR = reinterpret_cast<float*>(smem + DQ_NST * DQ_STAGE_B);   // [E][BT]
 
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
         const long roff = (long)bc * JB * DH;
 #pragma unroll
         for (int k = 0; k < FILL; ++k) {
-            const int id = wave + 4 * k;             // 0..23: tile id/8 (K, U, V), 4-row group id%8
+            const int id = wave + NW * k;            // 0..23: tile id/8 (K, U, V), 4-row group id%8
             const int which = id >> 3;
             const long toff = which == 0 ? 0 : (which == 1 ? offU : offV);
             tile_fill_ins<DH>(Kh + toff + roff, DH, st + which * TILE_B, id & 7, lane);
@@ -81,7 +82,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
             go[ct][ks] = *reinterpret_cast<const bf16x8*>(gr + ks * 16);
         }
     }
-    for (int idx = tid; idx < BT * p.E; idx += 256) {
+    for (int idx = tid; idx < BT * p.E; idx += NTHR) {
         int t = tb * BT + idx / p.E;
         t = t < p.S ? t : p.S - 1;
         sR[(idx % p.E) * BT + idx / p.E] = p.R[(rowbase + t) * p.E + idx % p.E];
@@ -96,6 +97,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
             for (int x = 0; x < 16; ++x) dq[i][ct][x] = 0.0f;
 
     const int krow = row_perm32(l32);
+    const TrLane<CT> trl = make_tr_lane<CT, 8, 4>(lane);
     int blk = 0;
     for (int e = 0; e < p.E; ++e) {
         float dr[NCT];
@@ -149,18 +151,34 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dqdr_kernel(DqArgs p)
                         dmt[ct][s][kk] = (bf16_t)((r[ct] * a) * (nn * w));
                     }
 
-#pragma unroll
-            for (int i = 0; i < CT; ++i)
-#pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    const bf16x8 akt = tile_read_cols(sK, i, 16 * s + 8 * g, 16 * s + 8 * g + 4, lane);
-                    const bf16x8 aut = tile_read_cols(sU, i, 16 * s + 8 * g, 16 * s + 8 * g + 4, lane);
+            // second products: operand pairs (Kt, Ut) are requested two steps ahead of the MFMAs that consume them; the
+            // region is fenced so that the partial LDS waits below count exactly these reads
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                constexpr int NSET = 2 * CT;          // (s, i) in s-major order
+                TrOperand tk[3], tu[3];
+                auto request = [&](auto ic) {
+                    constexpr int idx = decltype(ic)::value;
+                    constexpr int s = idx / CT, i = idx % CT;
+                    tk[idx % 3] = tile_read_cols_async<4096 * s>(lds_addr(sK), trl, i);
+                    tu[idx % 3] = tile_read_cols_async<4096 * s + TILE_B>(lds_addr(sK), trl, i);
+                };
+                request(std::integral_constant<int, 0>{});
+                request(std::integral_constant<int, 1>{});
+                static_for<NSET>([&](auto ic) {
+                    constexpr int idx = decltype(ic)::value;
+                    constexpr int s = idx / CT, i = idx % CT;
+                    if constexpr (idx + 2 < NSET) request(std::integral_constant<int, idx + 2>{});
+                    constexpr int ahead = (NSET - 1 - idx) < 2 ? (NSET - 1 - idx) : 2;
+                    lds_tr_wait_n<4 * ahead>(tk[idx % 3], tu[idx % 3]);
 #pragma unroll
                     for (int ct = 0; ct < NCT; ++ct) {
-                        dq[i][ct] = mfma32(akt, dmt[ct][s], dq[i][ct]);
-                        dq[i][ct] = mfma32(aut, dnt[ct][s], dq[i][ct]);
+                        dq[i][ct] = mfma32(tr_value(tk[idx % 3]), dmt[ct][s], dq[i][ct]);
+                        dq[i][ct] = mfma32(tr_value(tu[idx % 3]), dnt[ct][s], dq[i][ct]);
                     }
-                }
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
         // dR[t, e]: the two lane halves hold disjoint j rows of the same token column.
 #pragma unroll
@@ -202,10 +220,11 @@ struct DwArgs {
     int B, H, G, S, E, nbe, nslice;
 };
 
-constexpr int DW_RTILE_B = 16 * 1024;                 // staged R tile: [E][32] fp32, E <= 128
+constexpr int DW_NST = 4;                              // LDS stages of the token-tile ring
+constexpr int DW_RTILE_B = 8 * 1024;                   // staged R tile: [E][32] fp32, E <= 64
 constexpr int DW_STAGE_B = 2 * TILE_B + DW_RTILE_B;    // Q tile | dO tile | R tile
 
-template <int DH>
+template <int DH, bool TAIL>
 __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
 {
     constexpr int KS = DH / 16, CT = DH / 32;
@@ -222,12 +241,21 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     const int e_w = jb_c / p.nbe;
     const long wrow = ((long)hk * nblk + jb_c) * JB + l32;      // this lane's row of K/U/V (column j of the products)
 
-    bf16x8 kB[KS], uB[KS], vB[KS];
+    // K and U blocks stay in (accumulation) registers as MFMA B operands for the whole kernel; the V block of each
+    // wave is parked in LDS (one swizzled tile per wave, behind the ring) and re-read every tile.
+    unsigned char* sVw = smem_raw + DW_NST * DW_STAGE_B + wave * TILE_B;
+    float* sZero = reinterpret_cast<float*>(smem_raw + DW_NST * DW_STAGE_B + 4 * TILE_B);   // 32 zero gate values
+    if (tid < 32) sZero[tid] = 0.0f;
+    {
+        const bf16_t* vblk = p.V + (((long)hk * nblk + jb_c) * JB) * DH;
+#pragma unroll
+        for (int ins = 0; ins < 8; ++ins) tile_fill_ins<DH>(vblk, DH, sVw, ins, lane);
+    }
+    bf16x8 kB[KS], uB[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         kB[ks] = *reinterpret_cast<const bf16x8*>(p.K + wrow * DH + ks * 16 + 8 * g);
         uB[ks] = *reinterpret_cast<const bf16x8*>(p.U + wrow * DH + ks * 16 + 8 * g);
-        vB[ks] = *reinterpret_cast<const bf16x8*>(p.V + wrow * DH + ks * 16 + 8 * g);
     }
 
     f32x16 dk[CT], du[CT], dv[CT];
@@ -239,11 +267,14 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     const int nS = (p.S + 31) / 32;
     const int ntile = p.G * p.B * nS;
     const int t_begin = (int)((long)ntile * z / p.nslice), t_end = (int)((long)ntile * (z + 1) / p.nslice);
+    const int nt = t_end - t_begin;
 
     // Tile cursor of the prefetcher: tile index -> (q-head of the group, batch, 32-token tile), advanced incrementally.
     int pf_st = t_begin % nS, pf_bb = (t_begin / nS) % p.B, pf_gi = t_begin / (nS * p.B);
+    int pf_left = nt;                                 // tiles not yet requested
 
-    // per-lane constants of the tile fill: this wave's two 4-row groups, swizzled source chunk
+    // per-lane constants of the tile fill: this wave's two 4-row groups of the Q/dO tiles (swizzled source chunk)
+    constexpr int RINS = 8;                           // R-tile instructions per wave: covers E <= 64 with 4 waves
     int fill_row[2], fill_coff[2];
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
@@ -252,38 +283,46 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         int c = (lane & 15) ^ swz16(r);
         c = c < NCHUNK ? c : 0;                       // unused chunk positions of narrow rows load a dummy chunk
         fill_row[k] = r;
-        fill_coff[k] = c * 8;
+        fill_coff[k] = c * 16;                        // bytes
     }
 
-    // Asynchronous fill of stage `sidx` with the tile under the cursor; every wave issues its share of LDS-direct
-    // loads (no staging registers), then the cursor advances.  Rows past the end of a sequence are clamped to its last
-    // row and their gate value is zeroed afterwards (zero_tail), which removes them from all three products.
-    auto issue_tile = [&](int sidx) {
-        const long rb = ((long)pf_bb * p.H + hk * p.G + pf_gi) * p.S;
-        const int t0 = pf_st * 32;
+    // Asynchronous fill of stage `sidx` with the tile under the cursor (nothing once all tiles are requested); every wave
+    // issues its share of LDS-direct loads (no staging registers), then the cursor advances.  Addresses are a
+    // wave-uniform 64-bit base plus a 32-bit lane offset.  Rows past the end of a sequence are clamped to its last row
+    // and their gate value is zeroed afterwards (zero_tail), which removes them from all three products.
+    // Returns the number of valid rows of the tile (32 unless it is a tail tile).
+    auto issue_tile = [&](int sidx) -> int {
+        const long rb = ((long)pf_bb * p.H + hk * p.G + pf_gi) * p.S + pf_st * 32;   // first token row of the tile
+        const int last = p.S - pf_st * 32 - 1;                                       // last valid row of the tile (>= 0)
+        const char* qb = reinterpret_cast<const char*>(p.Q + rb * DH);
+        const char* gb = reinterpret_cast<const char*>(p.dO + rb * DH);
+        const char* rbp = reinterpret_cast<const char*>(p.R + rb * p.E);
         unsigned char* sbase = smem_raw + sidx * DW_STAGE_B;
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
-            int t = t0 + fill_row[k];
-            t = t < p.S ? t : p.S - 1;
-            const long off = (rb + t) * DH + fill_coff[k];
+            const int row = TAIL ? (fill_row[k] < last ? fill_row[k] : last) : fill_row[k];
+            const unsigned off = (unsigned)(row * (DH * 2) + fill_coff[k]);
             const int ins = wave + 4 * k;
-            __builtin_amdgcn_global_load_lds((gptr_t)(p.Q + off), (lptr_t)(sbase + ins * 1024), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gptr_t)(p.dO + off), (lptr_t)(sbase + TILE_B + ins * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(qb + off), (lptr_t)(sbase + ins * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(gb + off), (lptr_t)(sbase + TILE_B + ins * 1024), 16, 0, 0);
         }
-        // R tile: [E][32] fp32, one 4-byte element per lane, two experts per instruction.
+        // R tile: [E][32] fp32, one 4-byte element per lane, two experts per instruction; experts past E reload the last.
+        const int trow = TAIL ? (l32 < last ? l32 : last) : l32;
         for (int ins = wave; 2 * ins < p.E; ins += 4) {
             int e = 2 * ins + (lane >> 5);
             e = e < p.E ? e : p.E - 1;
-            int t = t0 + l32;
-            t = t < p.S ? t : p.S - 1;
-            __builtin_amdgcn_global_load_lds((gptr_t)(p.R + (rb + t) * p.E + e),
-                                             (lptr_t)(sbase + 2 * TILE_B + ins * 256), 4, 0, 0);
+            const unsigned off = (unsigned)((trow * p.E + e) * 4);
+            __builtin_amdgcn_global_load_lds((gptr_t)(rbp + off), (lptr_t)(sbase + 2 * TILE_B + ins * 256), 4, 0, 0);
         }
-        if (++pf_st == nS) {
-            pf_st = 0;
-            if (++pf_bb == p.B) { pf_bb = 0; ++pf_gi; }
-        }
+        // advance unless this was the last tile of the slice (then later requests reload it, harmlessly)
+        const bool more = pf_left > 1;
+        pf_left -= more ? 1 : 0;
+        const bool wrap_s = more && (pf_st + 1 == nS);
+        pf_st = more ? (wrap_s ? 0 : pf_st + 1) : pf_st;
+        const bool wrap_b = wrap_s && (pf_bb + 1 == p.B);
+        pf_bb = wrap_s ? (wrap_b ? 0 : pf_bb + 1) : pf_bb;
+        pf_gi += wrap_b ? 1 : 0;
+        return last + 1;
     };
     // Called by every wave after its own loads of stage `sidx` have landed and before the barrier that publishes
     // the stage: zeroes the gate values of the rows a tail tile does not have.
@@ -293,78 +332,136 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
             if (l32 >= nvalid) sR[ins * 64 + lane] = 0.0f;
     };
 
-    int cur_st = pf_st;                                // 32-token tile index (within its sequence) of tile `tau`
-    if (t_begin < t_end) issue_tile(0);
-
     const int fr = swz16(l32);
-    f32x16 zero16;
-#pragma unroll
-    for (int x = 0; x < 16; ++x) zero16[x] = 0.0f;
+    const TrLane<CT> trl = make_tr_lane<CT, 4, 8>(lane);
+    const int rowoff = l32 * 256;
+    const int xg = (g ^ fr) << 4;                     // chunk byte offset of k-step 0; k-step ks is xg ^ (ks << 5)
 
-    auto process = [&](auto stage_c, int tau) {
-        constexpr int cur = decltype(stage_c)::value;
-        wait_vmcnt<0>();                      // this wave's share of stage `cur` has landed
-        const int nvalid = p.S - cur_st * 32;
-        if (nvalid < 32) zero_tail(cur, nvalid);
-        if (++cur_st == nS) cur_st = 0;
-        __syncthreads();                      // ... and everybody's; all waves are done reading the other stage
-        if (tau + 1 < t_end) issue_tile(cur ^ 1);
-
-        const unsigned char* sQ = smem_raw + cur * DW_STAGE_B;
+    // first products of the tile in stage ST -> (m, n, da) in architectural VGPRs, element-wise work of the PREVIOUS
+    // tile (registers pm, pn, pda; gate values from stage SP) dealt out between the k-steps so that the VALU works
+    // under the MFMAs; then the token contraction of the previous tile.
+    //   registers 4a+b of m/n/da: token 8a + 4g + b (rows), column j = l32.
+    auto step = [&](auto st_c, auto sp_c, f32x16& m, f32x16& n, f32x16& da, const f32x16& pm, const f32x16& pn,
+                    const f32x16& pda, bool live) {
+        constexpr int ST = decltype(st_c)::value, SP = decltype(sp_c)::value;
+        const unsigned char* sQ = smem_raw + ST * DW_STAGE_B;
         const unsigned char* sG = sQ + TILE_B;
-        const float* sR = reinterpret_cast<const float*>(sG + TILE_B) + e_w * 32;
+        const unsigned char* pQ = smem_raw + SP * DW_STAGE_B;
+        const unsigned char* pG = pQ + TILE_B;
+        // the previous tile's gate values, or zeros when there is no previous tile to contract (first step of a slice,
+        // phantom steps that pad the loop): a zero gate makes P, dM and dN exactly zero
+        const float* pR = live ? reinterpret_cast<const float*>(pG + TILE_B) + e_w * 32 : sZero;
 
-        f32x16 m, n, da;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const int off = l32 * 256 + (((2 * ks + g) ^ fr) << 4);
-            const bf16x8 aq = *reinterpret_cast<const bf16x8*>(sQ + off);
-            const bf16x8 ag = *reinterpret_cast<const bf16x8*>(sG + off);
-            m = mfma32(aq, kB[ks], ks == 0 ? zero16 : m);
-            n = mfma32(aq, uB[ks], ks == 0 ? zero16 : n);
-            da = mfma32(ag, vB[ks], ks == 0 ? zero16 : da);
-        }
-
-        // registers 4a+b of m/n/da are token 8a + 4g + b (rows), column j = l32.
         bf16x8 pB[2], dmB[2], dnB[2];
-#pragma unroll
-        for (int a = 0; a < 4; ++a) {
-            const f32x4 rv = *reinterpret_cast<const f32x4*>(sR + 8 * a + 4 * g);
-#pragma unroll
-            for (int bb = 0; bb < 4; ++bb) {
-                const int i = 4 * a + bb;
-                const float x = m[i], nn = n[i], dA = da[i], rr = rv[bb];
-                const float sg = fast_sigmoid(x);
-                const float sl = x * sg;                               // silu(m)
-                const float w = __builtin_fmaf(sl, 1.0f - sg, sg);     // silu'(m)
-                const float rs = rr * sl;
-                pB[i >> 3][i & 7] = (bf16_t)(rs * nn);
-                dnB[i >> 3][i & 7] = (bf16_t)(rs * dA);
-                dmB[i >> 3][i & 7] = (bf16_t)((rr * w) * (nn * dA));
+        bf16x8 aq[2], ag[2], vB[2];
+        aq[0] = *reinterpret_cast<const bf16x8*>(sQ + rowoff + xg);
+        ag[0] = *reinterpret_cast<const bf16x8*>(sG + rowoff + xg);
+        vB[0] = *reinterpret_cast<const bf16x8*>(sVw + rowoff + xg);
+        f32x4 rv;
+        static_for<KS>([&](auto kc) {
+            constexpr int ks = decltype(kc)::value;
+            if constexpr (ks + 1 < KS) {
+                const int off = rowoff + (xg ^ ((ks + 1) << 5));
+                aq[(ks + 1) & 1] = *reinterpret_cast<const bf16x8*>(sQ + off);
+                ag[(ks + 1) & 1] = *reinterpret_cast<const bf16x8*>(sG + off);
+                vB[(ks + 1) & 1] = *reinterpret_cast<const bf16x8*>(sVw + off);
             }
-        }
+            // One MFMA, then one element of the previous tile's element-wise work, and so on: back-to-back MFMAs would
+            // block this wave's (in-order) instruction stream until the matrix pipe accepts each of them.
+            auto element = [&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                if constexpr (i < 16) {
+                    if constexpr ((i & 3) == 0) rv = *reinterpret_cast<const f32x4*>(pR + 8 * (i >> 2) + 4 * g);
+                    const float x = pm[i], nn = pn[i], dA = pda[i], rr = rv[i & 3];
+                    const float sg = fast_sigmoid(x);
+                    const float sl = x * sg;                               // silu(m)
+                    const float w = __builtin_fmaf(sl, 1.0f - sg, sg);     // silu'(m)
+                    const float rs = rr * sl;
+                    pB[i >> 3][i & 7] = (bf16_t)(rs * nn);
+                    dnB[i >> 3][i & 7] = (bf16_t)(rs * dA);
+                    dmB[i >> 3][i & 7] = (bf16_t)((rr * w) * (nn * dA));
+                }
+            };
+            constexpr int EPK = (16 + KS - 1) / KS;   // elements per k-step (2 for d_h = 128)
+            if constexpr (ks == 0) mfma32_vgpr_first_bacc(m, aq[0], kB[0]);
+            else mfma32_vgpr_acc_bacc(m, aq[ks & 1], kB[ks]);
+            element(std::integral_constant<int, EPK * ks>{});
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (ks == 0) mfma32_vgpr_first_bacc(n, aq[0], uB[0]);
+            else mfma32_vgpr_acc_bacc(n, aq[ks & 1], uB[ks]);
+            if constexpr (EPK > 1) element(std::integral_constant<int, EPK * ks + 1>{});
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (ks == 0) mfma32_vgpr_first(da, ag[0], vB[0]);
+            else mfma32_vgpr_acc(da, ag[ks & 1], vB[ks & 1]);
+            static_for<(EPK > 2 ? EPK - 2 : 0)>(
+                [&](auto dc) { element(std::integral_constant<int, EPK * ks + 2 + decltype(dc)::value>{}); });
+            __builtin_amdgcn_sched_barrier(0);
+        });
 
-        // token contraction: A = Q^T / dO^T gathered from the row-major tiles with transposing LDS reads.
-        // k-slot (s, g, kk) of the B operands is token 16s + 8(kk/4) + 4g + kk%4; a 16-lane group covers 16 columns c.
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                const bf16x8 aqt = tile_read_cols(sQ, ct, 16 * s + 4 * g, 16 * s + 4 * g + 8, lane);
-                const bf16x8 agt = tile_read_cols(sG, ct, 16 * s + 4 * g, 16 * s + 4 * g + 8, lane);
-                dk[ct] = mfma32(aqt, dmB[s], dk[ct]);
-                du[ct] = mfma32(aqt, dnB[s], du[ct]);
-                dv[ct] = mfma32(agt, pB[s], dv[ct]);
-            }
+        // token contraction of the previous tile: A = Q^T / dO^T gathered from the row-major tiles with transposing LDS
+        // reads.  k-slot (s, g, kk) of the B operands is token 16s + 8(kk/4) + 4g + kk%4; a 16-lane group covers 16
+        // columns c.
+        __builtin_amdgcn_sched_barrier(0);
+        {
+            constexpr int NSET = 2 * CT;              // (ct, s) in ct-major order
+            TrOperand tq[3], tg[3];
+            auto request = [&](auto ic) {
+                constexpr int idx = decltype(ic)::value;
+                constexpr int ct = idx / 2, s = idx % 2;
+                tq[idx % 3] = tile_read_cols_async<4096 * s>(lds_addr(pQ), trl, ct);
+                tg[idx % 3] = tile_read_cols_async<4096 * s + TILE_B>(lds_addr(pQ), trl, ct);
+            };
+            request(std::integral_constant<int, 0>{});
+            request(std::integral_constant<int, 1>{});
+            static_for<NSET>([&](auto ic) {
+                constexpr int idx = decltype(ic)::value;
+                constexpr int ct = idx / 2, s = idx % 2;
+                if constexpr (idx + 2 < NSET) request(std::integral_constant<int, idx + 2>{});
+                constexpr int ahead = (NSET - 1 - idx) < 2 ? (NSET - 1 - idx) : 2;
+                lds_tr_wait_n<4 * ahead>(tq[idx % 3], tg[idx % 3]);
+                dk[ct] = mfma32(tr_value(tq[idx % 3]), dmB[s], dk[ct]);
+                du[ct] = mfma32(tr_value(tq[idx % 3]), dnB[s], du[ct]);
+                dv[ct] = mfma32(tr_value(tg[idx % 3]), pB[s], dv[ct]);
+            });
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_result_fence(m, n, da);
     };
 
-    // two tiles per trip so that the LDS stage (and every LDS address) is a compile-time constant
-    int tau = t_begin;
-    for (; tau + 1 < t_end; tau += 2) {
-        process(std::integral_constant<int, 0>{}, tau);
-        process(std::integral_constant<int, 1>{}, tau + 1);
+    // Pipeline over tiles k = 0 .. nt (step k: first products of tile k, element-wise + contraction of tile k-1).
+    // Stage of tile k is k % 4; the two (m, n, da) register sets alternate with the parity of k.  Before step k every
+    // wave waits for its own outstanding loads (tiles <= k), then the barrier publishes tile k and retires the stage
+    // that tile k+2 is about to overwrite (last read by the contraction of tile k-2 in step k-1).
+    f32x16 mA, nA, dA_, mB, nB, dB_;
+#pragma unroll
+    for (int x = 0; x < 16; ++x) { mA[x] = 0.0f; nA[x] = 0.0f; dA_[x] = 0.0f; mB[x] = 0.0f; nB[x] = 0.0f; dB_[x] = 0.0f; }
+    int nv0 = issue_tile(0), nv1 = issue_tile(1), nv2 = 32, nv3 = 32;   // valid rows of the tile in each stage
+    auto sync_step = [&](auto st_c, int nvalid, int& nv_next) {
+        constexpr int ST = decltype(st_c)::value;
+        wait_vmcnt<0>();
+        if constexpr (TAIL) {
+            if (nvalid < 32) zero_tail(ST, nvalid);
+        }
+        __syncthreads();
+        nv_next = issue_tile((ST + 2) % DW_NST);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    // nt + 1 steps are needed (step k contracts tile k-1); the count is padded to a multiple of 4 with phantom steps
+    // whose products are computed on whatever the stage holds and contracted with a zero gate.
+    for (int k = 0; k <= nt; k += 4) {
+        sync_step(I0{}, nv0, nv2);
+        step(I0{}, I3{}, mA, nA, dA_, mB, nB, dB_, k > 0);
+        sync_step(I1{}, nv1, nv3);
+        step(I1{}, I0{}, mB, nB, dB_, mA, nA, dA_, k < nt);
+        sync_step(I2{}, nv2, nv0);
+        step(I2{}, I1{}, mA, nA, dA_, mB, nB, dB_, k + 1 < nt);
+        sync_step(I3{}, nv3, nv1);
+        step(I3{}, I2{}, mB, nB, dB_, mA, nA, dA_, k + 2 < nt);
     }
-    if (tau < t_end) process(std::integral_constant<int, 0>{}, tau);
+    wait_vmcnt<0>();
 
     if (active) {
         // dK^T registers 4a+b of row tile ct: c = 32ct + 8a + 4g + b, column j = l32 -> 16-byte runs along c.
@@ -432,7 +529,11 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
                                const void* dO, void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32,
                                void* ws, const Dims& d, hipStream_t st, int phases)
 {
-    constexpr int NCT = 2;
+#ifndef DQ_VARIANT
+#define DQ_VARIANT 1, 8
+#endif
+    constexpr int DQV[2] = {DQ_VARIANT};
+    constexpr int NCT = DQV[0], NW = DQV[1];
     hipError_t err = hipSuccess;
     float* part = reinterpret_cast<float*>(ws);
     const int nbe = d.d_e / JB, G = d.H / d.Hkuv;
@@ -440,18 +541,18 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
     if (phases & 2) {
         DqArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R,
                  (bf16_t*)dQ, dR, d.H, G, d.S, d.E, nbe};
-        const int tokw = 128 * NCT;
+        const int tokw = NW * 32 * NCT;
         const int smem = DQ_NST * DQ_STAGE_B + d.E * tokw * (int)sizeof(float);
         if (smem > 160 * 1024) return hipErrorInvalidValue;
         static int attr_smem = 0;   // dynamic LDS above 64 KB must be opted into, per kernel
         if (smem > attr_smem) {
-            err = hipFuncSetAttribute((const void*)mhffn_bwd_dqdr_kernel<DH, NCT>,
+            err = hipFuncSetAttribute((const void*)mhffn_bwd_dqdr_kernel<DH, NCT, NW>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
             if (err != hipSuccess) return err;
             attr_smem = smem;
         }
         dim3 grid((unsigned)d.H, (unsigned)((d.S + tokw - 1) / tokw), (unsigned)d.B);
-        hipLaunchKernelGGL((mhffn_bwd_dqdr_kernel<DH, NCT>), grid, dim3(256), smem, st, a);
+        hipLaunchKernelGGL((mhffn_bwd_dqdr_kernel<DH, NCT, NW>), grid, dim3(NW * 64), smem, st, a);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }
@@ -459,11 +560,24 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
     if (phases & 4) {
         DwArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, part,
                  d.B, d.H, G, d.S, d.E, nbe, nslice};
-        const int smem = 2 * DW_STAGE_B;
-        if (d.E > 128) return hipErrorInvalidValue;   // staged R tile holds at most 128 experts
+        const int smem = DW_NST * DW_STAGE_B + 4 * TILE_B + 128;
+        static bool attr_done = false;   // dynamic LDS above 64 KB must be opted into, per kernel
+        if (!attr_done) {
+            err = hipFuncSetAttribute((const void*)mhffn_bwd_dkdudv_kernel<DH, false>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+            if (err == hipSuccess)
+                err = hipFuncSetAttribute((const void*)mhffn_bwd_dkdudv_kernel<DH, true>,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+            if (err != hipSuccess) return err;
+            attr_done = true;
+        }
+        if (d.E > 64) return hipErrorInvalidValue;   // staged R tile holds at most 64 experts
         const int nblk = d.E * nbe;
         dim3 grid((unsigned)((nblk + 3) / 4), (unsigned)d.Hkuv, (unsigned)nslice);
-        hipLaunchKernelGGL((mhffn_bwd_dkdudv_kernel<DH>), grid, dim3(256), smem, st, a);
+        if (d.S % 32 == 0)
+            hipLaunchKernelGGL((mhffn_bwd_dkdudv_kernel<DH, false>), grid, dim3(256), smem, st, a);
+        else
+            hipLaunchKernelGGL((mhffn_bwd_dkdudv_kernel<DH, true>), grid, dim3(256), smem, st, a);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }

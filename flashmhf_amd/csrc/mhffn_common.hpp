@@ -72,6 +72,37 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c)
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
+// The same instruction with its accumulator forced into architectural VGPRs (the compiler picks one register file for
+// the accumulators of all builtin MFMAs of a kernel; a one-wave-per-SIMD kernel gets AGPRs, from which every value the
+// VALU needs costs a v_accvgpr_read).  Used for products whose result feeds element-wise VALU work directly.
+// The compiler cannot see that this is an MFMA, so the caller must leave the required wait states between the last of
+// these and the first VALU read of the result (mfma_result_fence).  A/B operand waits (LDS loads) are still inserted
+// by the compiler, back-to-back accumulation into the same registers is interlocked by hardware.
+__device__ __forceinline__ void mfma32_vgpr_first(f32x16& d, bf16x8 a, bf16x8 b)
+{
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma32_vgpr_acc(f32x16& d, bf16x8 a, bf16x8 b)
+{
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+}
+// Same, with the B operand held in an accumulation register (AGPRs are legal MFMA A/B sources): used for operands that
+// stay resident for a whole kernel, so they do not compete with the VALU's working set for architectural VGPRs.
+__device__ __forceinline__ void mfma32_vgpr_first_bacc(f32x16& d, bf16x8 a, bf16x8 b)
+{
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+}
+__device__ __forceinline__ void mfma32_vgpr_acc_bacc(f32x16& d, bf16x8 a, bf16x8 b)
+{
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+}
+__device__ __forceinline__ void mfma_result_fence(f32x16& a, f32x16& b, f32x16& c)
+{
+    // 8-pass MFMA result -> VALU read needs at most 18 wait states on gfx940-class hardware; leave 32.  The results
+    // are operands of the statement, so no read of them can be scheduled above it.
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(a), "+v"(b), "+v"(c));
+}
+
 __device__ __forceinline__ float fast_sigmoid(float x)
 {
     // 1 / (1 + 2^(-x log2 e)): v_mul, v_exp_f32, v_add, v_rcp_f32.  x -> -inf gives rcp(inf) = 0, x -> +inf gives 1.
@@ -116,20 +147,82 @@ __device__ __forceinline__ bf16x8 tile_read_rows(const unsigned char* tile, int 
 // A operand (32 rows = tile columns 32ct + l32, 16 k = tile rows) from a swizzled tile, transposed use:
 // lane holds column 32ct + l32; its 8 k values are tile rows rlo + {0..3} then rhi + {0..3}.  rlo/rhi must be uniform
 // within each 16-lane group (they may depend on lane / 32).
-__device__ __forceinline__ bf16x8 tile_read_cols(const unsigned char* tile, int ct, int rlo, int rhi, int lane)
+//
+// The two ds_read_b64_tr_b16 are issued from inline assembly, not through the compiler builtin: behind the builtin the
+// compiler cannot tell that the read does not touch the LDS stage an asynchronous LDS-direct load is filling, and puts
+// a full s_waitcnt vmcnt(0) in front of it, which stalls every loop iteration for the whole global-memory latency.
+// The price is that the compiler does not know these reads are in flight either: the consumer must call
+// lds_tr_wait() on the operands before their first use.
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+struct TrOperand {
+    u32x2 lo, hi;
+};
+__device__ __forceinline__ unsigned lds_addr(const void* p)
 {
-    typedef __attribute__((address_space(3))) v4bf16_t* lds_v4_ptr;
-    const int lam = lane & 15, l32 = lane & 31;
-    const int chunk = 4 * ct + 2 * (l32 >> 4) + ((lam & 3) >> 1);
-    const int r0 = rlo + (lam >> 2), r1 = rhi + (lam >> 2);
-    const unsigned char* p0 = tile + r0 * TILE_ROW_B + ((chunk ^ swz16(r0)) << 4) + (lam & 1) * 8;
-    const unsigned char* p1 = tile + r1 * TILE_ROW_B + ((chunk ^ swz16(r1)) << 4) + (lam & 1) * 8;
-    v4bf16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4_ptr)(p0));
-    v4bf16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4_ptr)(p1));
-    bf16x8 r;
-    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
-    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
-    return r;
+    return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+// Per-lane byte offsets (inside a tile, for s = 0) of the two reads of a transposed operand, for every column tile ct.
+// The tile rows a lane group reads are  16 s + RG * (lane / 32) + RH * hi + (lane % 16) / 4,  hi = 0, 1
+//   (RG, RH) = (8, 4): k-slot (s, g, kk) is row 16 s + 8 g + kk            (weights: second products of fwd, dQ)
+//   (RG, RH) = (4, 8): k-slot (s, g, kk) is row 16 s + 8 (kk / 4) + 4 g + kk % 4   (tokens: dK/dU/dV contraction)
+// s only adds 16 rows = 4096 bytes (the swizzle has period 16 rows), which goes into the instruction's immediate offset.
+template <int CT>
+struct TrLane {
+    unsigned off[CT][2];
+};
+template <int CT, int RG, int RH>
+__device__ __forceinline__ TrLane<CT> make_tr_lane(int lane)
+{
+    TrLane<CT> t;
+    const int lam = lane & 15, l32 = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi) {
+            const int r = RG * g + RH * hi + (lam >> 2);
+            const int chunk = 4 * ct + 2 * (l32 >> 4) + ((lam & 3) >> 1);
+            t.off[ct][hi] = r * TILE_ROW_B + ((chunk ^ swz16(r)) << 4) + (lam & 1) * 8;
+        }
+    return t;
+}
+// Requests operand (ct, s) of the tile at LDS byte address `tile_addr` (wave-uniform); IMM = 4096 * s + any
+// compile-time displacement (must stay below 65536 together).
+template <int IMM, int CT>
+__device__ __forceinline__ TrOperand tile_read_cols_async(unsigned tile_addr, const TrLane<CT>& tl, int ct)
+{
+    const unsigned a0 = tile_addr + tl.off[ct][0], a1 = tile_addr + tl.off[ct][1];
+    TrOperand t;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(t.lo) : "v"(a0), "n"(IMM));
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(t.hi) : "v"(a1), "n"(IMM));
+    return t;
+}
+// Waits for every LDS operation of this wave (lgkmcnt(0)); the operands are inputs and outputs of the statement, so no
+// use of them can be scheduled above it.
+__device__ __forceinline__ void lds_tr_wait(TrOperand& a)
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.lo), "+v"(a.hi));
+}
+__device__ __forceinline__ void lds_tr_wait(TrOperand& a, TrOperand& b)
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.lo), "+v"(a.hi), "+v"(b.lo), "+v"(b.hi));
+}
+__device__ __forceinline__ void lds_tr_wait(TrOperand& a, TrOperand& b, TrOperand& c, TrOperand& d)
+{
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(a.lo), "+v"(a.hi), "+v"(b.lo), "+v"(b.hi), "+v"(c.lo), "+v"(c.hi), "+v"(d.lo), "+v"(d.hi));
+}
+// Partial wait: at most N LDS operations of this wave still outstanding.  Only exact inside a region that the caller
+// has fenced with sched_barrier(0) and that contains no other LDS instruction than the asynchronous reads above
+// (LDS operations complete in order; each TrOperand is two of them).
+template <int N>
+__device__ __forceinline__ void lds_tr_wait_n(TrOperand& a, TrOperand& b)
+{
+    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a.lo), "+v"(a.hi), "+v"(b.lo), "+v"(b.hi) : "n"(N));
+}
+__device__ __forceinline__ bf16x8 tr_value(const TrOperand& t)
+{
+    u32x4 v = {t.lo[0], t.lo[1], t.hi[0], t.hi[1]};
+    return __builtin_bit_cast(bf16x8, v);
 }
 
 // s_waitcnt vmcnt(N) only (gfx9 encoding: vmcnt[3:0] at bits 3:0, vmcnt[5:4] at bits 15:14; other counters unconstrained).

@@ -96,6 +96,7 @@ __global__ __launch_bounds__(NW * 64) void mhffn_fwd_kernel(FwdArgs p)
             for (int x = 0; x < 16; ++x) oacc[i][ct][x] = 0.0f;
 
     const int krow = row_perm32(l32);   // K/U row fed as MFMA A-row l32 (see mhffn_common.hpp)
+    const TrLane<CT> trl = make_tr_lane<CT, 8, 4>(lane);
 
     auto gemm1 = [&](const unsigned char* st, f32x16 (&m)[NCT], f32x16 (&n)[NCT]) {
 #pragma unroll
@@ -145,7 +146,10 @@ __global__ __launch_bounds__(NW * 64) void mhffn_fwd_kernel(FwdArgs p)
         for (int i = 0; i < CT; ++i)
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                const bf16x8 av = tile_read_cols(st_cur + 2 * TILE_B, i, 16 * s + 8 * g, 16 * s + 8 * g + 4, lane);
+                TrOperand avo = s == 0 ? tile_read_cols_async<0>(lds_addr(st_cur + 2 * TILE_B), trl, i)
+                                       : tile_read_cols_async<4096>(lds_addr(st_cur + 2 * TILE_B), trl, i);
+                lds_tr_wait(avo);
+                const bf16x8 av = tr_value(avo);
 #pragma unroll
                 for (int ct = 0; ct < NCT; ++ct) oacc[i][ct] = mfma32(av, pt[ct][s], oacc[i][ct]);
             }
@@ -186,12 +190,13 @@ __global__ __launch_bounds__(NW * 64) void mhffn_fwd_kernel(FwdArgs p)
             float r[NCT];
 #pragma unroll
             for (int ct = 0; ct < NCT; ++ct) r[ct] = sR[e * BT + wave * (32 * NCT) + ct * 32 + l32];
-            bf16x8 av[CT][2];
+            TrOperand av[CT][2];
 #pragma unroll
             for (int i = 0; i < CT; ++i)
 #pragma unroll
                 for (int s = 0; s < 2; ++s)
-                    av[i][s] = tile_read_cols(sV, i, 16 * s + 8 * g, 16 * s + 8 * g + 4, lane);
+                    av[i][s] = s == 0 ? tile_read_cols_async<0>(lds_addr(sV), trl, i)
+                                      : tile_read_cols_async<4096>(lds_addr(sV), trl, i);
             __builtin_amdgcn_sched_barrier(0);
             bf16x8 pt[NCT][2];
 #pragma unroll
@@ -205,11 +210,13 @@ __global__ __launch_bounds__(NW * 64) void mhffn_fwd_kernel(FwdArgs p)
                     }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
+            for (int i = 0; i < CT; ++i) lds_tr_wait(av[i][0], av[i][1]);
+#pragma unroll
             for (int i = 0; i < CT; ++i)
 #pragma unroll
                 for (int s = 0; s < 2; ++s)
 #pragma unroll
-                    for (int ct = 0; ct < NCT; ++ct) oacc[i][ct] = mfma32(av[i][s], pt[ct][s], oacc[i][ct]);
+                    for (int ct = 0; ct < NCT; ++ct) oacc[i][ct] = mfma32(tr_value(av[i][s]), pt[ct][s], oacc[i][ct]);
             __builtin_amdgcn_sched_barrier(0);
         };
         f32x16 m[NCT], n[NCT];
