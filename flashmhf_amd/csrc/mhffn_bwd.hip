@@ -353,61 +353,85 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         const float* pR = live ? reinterpret_cast<const float*>(pG + TILE_B) + e_w * 32 : sZero;
 
         bf16x8 pB[2], dmB[2], dnB[2];
-        bf16x8 aq[2], ag[2], vB[2];
-        aq[0] = *reinterpret_cast<const bf16x8*>(sQ + rowoff + xg);
-        ag[0] = *reinterpret_cast<const bf16x8*>(sG + rowoff + xg);
-        vB[0] = *reinterpret_cast<const bf16x8*>(sVw + rowoff + xg);
-        f32x4 rv;
+        bf16x8 aq[3], ag[3], vB[3];                  // operand ring: k-step ks+2 is requested while ks is consumed
+#pragma unroll
+        for (int k0 = 0; k0 < 2; ++k0) {
+            const int off = rowoff + (xg ^ (k0 << 5));
+            aq[k0] = *reinterpret_cast<const bf16x8*>(sQ + off);
+            ag[k0] = *reinterpret_cast<const bf16x8*>(sG + off);
+            vB[k0] = *reinterpret_cast<const bf16x8*>(sVw + off);
+        }
+        // gate values of the previous tile for this lane's 16 token rows (4 consecutive rows per 16-byte read)
+        f32x4 rv[4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) rv[a] = *reinterpret_cast<const f32x4*>(pR + 8 * a + 4 * g);
+
+        // Element-wise work of the previous tile, one element (register index i of pm/pn/pda) at a time, in three slices
+        // of at most ~7 issue slots so that each fits under one MFMA (32 cycles): a = exp, b = sigmoid / silu,
+        // c = silu' and the three gated products.
+        float ev, sgv, slv;
+        auto ew_a = [&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            ev = __builtin_amdgcn_exp2f(-LOG2E * pm[i]);
+        };
+        auto ew_b = [&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            sgv = __builtin_amdgcn_rcpf(1.0f + ev);
+            slv = pm[i] * sgv;                              // silu(m)
+        };
+        auto ew_c = [&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            const float wv = __builtin_fmaf(slv, 1.0f - sgv, sgv);      // silu'(m)
+            const float nn = pn[i], dA = pda[i], rr = rv[i >> 2][i & 3];
+            const float rs = rr * slv;
+            pB[i >> 3][i & 7] = (bf16_t)(rs * nn);
+            dnB[i >> 3][i & 7] = (bf16_t)(rs * dA);
+            dmB[i >> 3][i & 7] = (bf16_t)((rr * wv) * (nn * dA));
+        };
+        auto ew_all = [&](auto ic) { ew_a(ic); ew_b(ic); ew_c(ic); };
+
+        // Phase 1: first products of this tile (24 MFMAs for d_h = 128) with elements 0..7 of the previous tile (the
+        // s = 0 operands of its contraction) dealt out between them.  One MFMA, then half an element, and so on:
+        // back-to-back MFMAs would block this wave's in-order instruction stream until the matrix pipe takes each.
+        constexpr int E1 = 8;                               // elements converted in phase 1
         static_for<KS>([&](auto kc) {
             constexpr int ks = decltype(kc)::value;
-            if constexpr (ks + 1 < KS) {
-                const int off = rowoff + (xg ^ ((ks + 1) << 5));
-                aq[(ks + 1) & 1] = *reinterpret_cast<const bf16x8*>(sQ + off);
-                ag[(ks + 1) & 1] = *reinterpret_cast<const bf16x8*>(sG + off);
-                vB[(ks + 1) & 1] = *reinterpret_cast<const bf16x8*>(sVw + off);
+            if constexpr (ks + 2 < KS) {
+                const int off = rowoff + (xg ^ ((ks + 2) << 5));
+                aq[(ks + 2) % 3] = *reinterpret_cast<const bf16x8*>(sQ + off);
+                ag[(ks + 2) % 3] = *reinterpret_cast<const bf16x8*>(sG + off);
+                vB[(ks + 2) % 3] = *reinterpret_cast<const bf16x8*>(sVw + off);
             }
-            // One MFMA, then one element of the previous tile's element-wise work, and so on: back-to-back MFMAs would
-            // block this wave's (in-order) instruction stream until the matrix pipe accepts each of them.
-            auto element = [&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                if constexpr (i < 16) {
-                    if constexpr ((i & 3) == 0) rv = *reinterpret_cast<const f32x4*>(pR + 8 * (i >> 2) + 4 * g);
-                    const float x = pm[i], nn = pn[i], dA = pda[i], rr = rv[i & 3];
-                    const float sg = fast_sigmoid(x);
-                    const float sl = x * sg;                               // silu(m)
-                    const float w = __builtin_fmaf(sl, 1.0f - sg, sg);     // silu'(m)
-                    const float rs = rr * sl;
-                    pB[i >> 3][i & 7] = (bf16_t)(rs * nn);
-                    dnB[i >> 3][i & 7] = (bf16_t)(rs * dA);
-                    dmB[i >> 3][i & 7] = (bf16_t)((rr * w) * (nn * dA));
-                }
-            };
-            constexpr int EPK = (16 + KS - 1) / KS;   // elements per k-step (2 for d_h = 128)
+            constexpr int e0 = ks * E1 / KS, e1 = (ks + 1) * E1 / KS;    // element(s) of this k-step (one for KS = 8)
             if constexpr (ks == 0) mfma32_vgpr_first_bacc(m, aq[0], kB[0]);
-            else mfma32_vgpr_acc_bacc(m, aq[ks & 1], kB[ks]);
-            element(std::integral_constant<int, EPK * ks>{});
+            else mfma32_vgpr_acc_bacc(m, aq[ks % 3], kB[ks]);
+            if constexpr (e1 > e0) ew_a(std::integral_constant<int, e0>{});
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (ks == 0) mfma32_vgpr_first_bacc(n, aq[0], uB[0]);
-            else mfma32_vgpr_acc_bacc(n, aq[ks & 1], uB[ks]);
-            if constexpr (EPK > 1) element(std::integral_constant<int, EPK * ks + 1>{});
+            else mfma32_vgpr_acc_bacc(n, aq[ks % 3], uB[ks]);
+            if constexpr (e1 > e0) ew_b(std::integral_constant<int, e0>{});
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (ks == 0) mfma32_vgpr_first(da, ag[0], vB[0]);
-            else mfma32_vgpr_acc(da, ag[ks & 1], vB[ks & 1]);
-            static_for<(EPK > 2 ? EPK - 2 : 0)>(
-                [&](auto dc) { element(std::integral_constant<int, EPK * ks + 2 + decltype(dc)::value>{}); });
+            else mfma32_vgpr_acc(da, ag[ks % 3], vB[ks % 3]);
+            if constexpr (e1 > e0) ew_c(std::integral_constant<int, e0>{});
+            static_for<(e1 - e0 > 1 ? e1 - e0 - 1 : 0)>([&](auto dc) {      // d_h < 128: more than one element per k-step
+                ew_all(std::integral_constant<int, e0 + 1 + decltype(dc)::value>{});
+            });
             __builtin_amdgcn_sched_barrier(0);
         });
 
-        // token contraction of the previous tile: A = Q^T / dO^T gathered from the row-major tiles with transposing LDS
-        // reads.  k-slot (s, g, kk) of the B operands is token 16s + 8(kk/4) + 4g + kk%4; a 16-lane group covers 16
-        // columns c.
+        // Phases 2 and 3: token contraction of the previous tile, s-major.  A = Q^T / dO^T gathered from the row-major
+        // tiles with transposing LDS reads (k-slot (s, g, kk) of the B operands is token 16s + 8(kk/4) + 4g + kk%4; a
+        // 16-lane group covers 16 columns c), requested two operand sets ahead.  The s = 0 MFMAs only need the operands
+        // phase 1 produced, so elements 8..15 are converted between them.  The region is fenced and contains no other
+        // LDS instruction, so the partial LDS waits count exactly the asynchronous reads.
         __builtin_amdgcn_sched_barrier(0);
         {
-            constexpr int NSET = 2 * CT;              // (ct, s) in ct-major order
+            constexpr int NSET = 2 * CT;              // (s, ct) in s-major order
             TrOperand tq[3], tg[3];
             auto request = [&](auto ic) {
                 constexpr int idx = decltype(ic)::value;
-                constexpr int ct = idx / 2, s = idx % 2;
+                constexpr int s = idx / CT, ct = idx % CT;
                 tq[idx % 3] = tile_read_cols_async<4096 * s>(lds_addr(pQ), trl, ct);
                 tg[idx % 3] = tile_read_cols_async<4096 * s + TILE_B>(lds_addr(pQ), trl, ct);
             };
@@ -415,13 +439,23 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
             request(std::integral_constant<int, 1>{});
             static_for<NSET>([&](auto ic) {
                 constexpr int idx = decltype(ic)::value;
-                constexpr int ct = idx / 2, s = idx % 2;
+                constexpr int s = idx / CT, ct = idx % CT;
                 if constexpr (idx + 2 < NSET) request(std::integral_constant<int, idx + 2>{});
                 constexpr int ahead = (NSET - 1 - idx) < 2 ? (NSET - 1 - idx) : 2;
                 lds_tr_wait_n<4 * ahead>(tq[idx % 3], tg[idx % 3]);
+                // elements of phase 2 handled around this operand set: (16 - E1) elements over CT sets
+                constexpr int f0 = E1 + ct * (16 - E1) / CT, f1 = E1 + (ct + 1) * (16 - E1) / CT;
                 dk[ct] = mfma32(tr_value(tq[idx % 3]), dmB[s], dk[ct]);
+                if constexpr (s == 0 && f1 > f0) ew_all(std::integral_constant<int, f0>{});
+                __builtin_amdgcn_sched_barrier(0);
                 du[ct] = mfma32(tr_value(tq[idx % 3]), dnB[s], du[ct]);
+                if constexpr (s == 0) {
+                    static_for<(f1 - f0 > 1 ? f1 - f0 - 1 : 0)>(
+                        [&](auto dc) { ew_all(std::integral_constant<int, f0 + 1 + decltype(dc)::value>{}); });
+                }
+                __builtin_amdgcn_sched_barrier(0);
                 dv[ct] = mfma32(tr_value(tg[idx % 3]), pB[s], dv[ct]);
+                __builtin_amdgcn_sched_barrier(0);
             });
         }
         __builtin_amdgcn_sched_barrier(0);
