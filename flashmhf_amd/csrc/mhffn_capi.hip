@@ -13,10 +13,13 @@ int check_dims_impl(const mhffn_dims* d, int dtype)
     if (d->B <= 0 || d->H <= 0 || d->Hkuv <= 0 || d->S <= 0 || d->E <= 0 || d->d_e <= 0 || d->d_h <= 0)
         return MHFFN_ERR_SHAPE;
     if (d->H % d->Hkuv != 0) return MHFFN_ERR_SHAPE;
-    if (d->E > 64) return MHFFN_ERR_SHAPE;   // the kernels stage a [E][256] fp32 gate tile in LDS next to the weight ring
-    if (dtype == MHFFN_DTYPE_F32) return MHFFN_ERR_DTYPE;   // no fp32 kernels in this build
-    if (d->d_h != 64 && d->d_h != 96 && d->d_h != 128) return MHFFN_ERR_HEAD_DIM;
-    if (d->d_e % 32 != 0) return MHFFN_ERR_EXPERT_DIM;
+    if (dtype == MHFFN_DTYPE_F32) {           // fp32 correctness path: generic tiles, no MFMA
+        if (d->d_h % 8 != 0 || d->d_h > 128) return MHFFN_ERR_HEAD_DIM;
+    } else {
+        if (d->E > 64) return MHFFN_ERR_SHAPE;   // the kernels stage a [E][256] fp32 gate tile in LDS next to the weight ring
+        if (d->d_h != 64 && d->d_h != 96 && d->d_h != 128) return MHFFN_ERR_HEAD_DIM;
+        if (d->d_e % 32 != 0) return MHFFN_ERR_EXPERT_DIM;
+    }
     // index arithmetic inside the kernels is 64-bit for rows, 32-bit for per-(b,h) token indices and grid extents
     if ((long long)d->B > 65535 || (long long)d->S > (1ll << 30)) return MHFFN_ERR_SHAPE;
     return MHFFN_OK;
@@ -33,10 +36,10 @@ const char* mhffn_strerror(int code)
     switch (code) {
         case MHFFN_OK: return "ok";
         case MHFFN_ERR_NULL_POINTER: return "null pointer argument";
-        case MHFFN_ERR_DTYPE: return "unsupported dtype (Q, K, U, V must be bfloat16; R float32)";
-        case MHFFN_ERR_HEAD_DIM: return "unsupported head dim (d_h must be 64, 96 or 128)";
-        case MHFFN_ERR_EXPERT_DIM: return "unsupported expert dim (d_e must be a multiple of 32)";
-        case MHFFN_ERR_SHAPE: return "invalid extents (all must be positive, H a multiple of Hkuv, E <= 64)";
+        case MHFFN_ERR_DTYPE: return "unsupported dtype (Q, K, U, V must all be bfloat16 or all float32; R float32)";
+        case MHFFN_ERR_HEAD_DIM: return "unsupported head dim (bf16: d_h must be 64, 96 or 128; fp32: a multiple of 8 up to 128)";
+        case MHFFN_ERR_EXPERT_DIM: return "unsupported expert dim (bf16: d_e must be a multiple of 32)";
+        case MHFFN_ERR_SHAPE: return "invalid extents (all must be positive, H a multiple of Hkuv; bf16: E <= 64)";
         case MHFFN_ERR_WORKSPACE: return "workspace missing or too small";
         case MHFFN_ERR_LAUNCH: return "kernel launch failed";
         case MHFFN_ERR_ALIGNMENT: return "pointer not 16-byte aligned";
@@ -46,6 +49,7 @@ const char* mhffn_strerror(int code)
 
 int mhffn_is_supported(int d_h, int d_e, int dtype)
 {
+    if (dtype == MHFFN_DTYPE_F32) return d_h > 0 && d_h % 8 == 0 && d_h <= 128 && d_e > 0;
     if (dtype != MHFFN_DTYPE_BF16) return 0;
     return (d_h == 64 || d_h == 96 || d_h == 128) && d_e > 0 && d_e % 32 == 0;
 }
@@ -55,12 +59,14 @@ int mhffn_check_dims(const mhffn_dims* dims, int dtype) { return check_dims_impl
 size_t mhffn_fwd_workspace_bytes(const mhffn_dims* dims, int dtype)
 {
     if (check_dims_impl(dims, dtype) != MHFFN_OK) return 0;
+    if (dtype == MHFFN_DTYPE_F32) return 0;
     return mhffn::fwd_workspace_bytes_bf16(to_dims(dims));
 }
 
 size_t mhffn_bwd_workspace_bytes(const mhffn_dims* dims, int dtype)
 {
     if (check_dims_impl(dims, dtype) != MHFFN_OK) return 0;
+    if (dtype == MHFFN_DTYPE_F32) return mhffn::bwd_workspace_bytes_f32(to_dims(dims));
     return mhffn::bwd_workspace_bytes_bf16(to_dims(dims));
 }
 
@@ -75,6 +81,10 @@ int mhffn_fwd_phases(const void* Q, const void* K, const void* U, const void* V,
         !aligned16(workspace))
         return MHFFN_ERR_ALIGNMENT;
     const mhffn::Dims d = to_dims(dims);
+    if (dtype == MHFFN_DTYPE_F32) {
+        if (!(phases & MHFFN_FWD_MAIN)) return MHFFN_OK;
+        return mhffn::launch_fwd_f32(Q, K, U, V, R, O, d, (hipStream_t)stream) == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
+    }
     const size_t need = mhffn::fwd_workspace_bytes_bf16(d);
     if (need > 0 && (!workspace || workspace_bytes < need)) return MHFFN_ERR_WORKSPACE;
     const hipError_t err = mhffn::launch_fwd_bf16(Q, K, U, V, R, O, workspace, d, (hipStream_t)stream, phases);
@@ -100,8 +110,13 @@ int mhffn_bwd_phases(const void* Q, const void* K, const void* U, const void* V,
     for (const void* p : ptrs)
         if (!aligned16(p)) return MHFFN_ERR_ALIGNMENT;
     const mhffn::Dims d = to_dims(dims);
-    const size_t need = mhffn::bwd_workspace_bytes_bf16(d);
+    const size_t need = dtype == MHFFN_DTYPE_F32 ? mhffn::bwd_workspace_bytes_f32(d) : mhffn::bwd_workspace_bytes_bf16(d);
     if (need > 0 && (!workspace || workspace_bytes < need)) return MHFFN_ERR_WORKSPACE;
+    if (dtype == MHFFN_DTYPE_F32)
+        return mhffn::launch_bwd_f32(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_dtype == MHFFN_DTYPE_F32, workspace, d,
+                                     (hipStream_t)stream, phases) == hipSuccess
+                   ? MHFFN_OK
+                   : MHFFN_ERR_LAUNCH;
     const hipError_t err = mhffn::launch_bwd_bf16(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR,
                                                   grad_w_dtype == MHFFN_DTYPE_F32, workspace, d, (hipStream_t)stream,
                                                   phases);

@@ -245,4 +245,12 @@ hipError_t launch_bwd_bf16(const void* Q, const void* K, const void* U, const vo
                            void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32,
                            void* ws, const Dims& d, hipStream_t st, int phases);
 
+// fp32 instantiation (mhffn_f32.hip): d_h a multiple of 8 up to 128, any d_e, any E.
+size_t bwd_workspace_bytes_f32(const Dims& d);
+hipError_t launch_fwd_f32(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
+                          const Dims& d, hipStream_t st);
+hipError_t launch_bwd_f32(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
+                          void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32, void* ws, const Dims& d,
+                          hipStream_t st, int phases);
+
 }  // namespace mhffn

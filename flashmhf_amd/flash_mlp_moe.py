@@ -6,7 +6,7 @@
 
 Same call signature, tensor contract, saved tensors (Q, K, U, V, R only -- no activations) and exception types.
 Differences, all widening: d_e may be any multiple of 32 (the reference needs 64, :758), the sequence length is
-free, and R's gradient is exact fp32 instead of bf16-rounded (:542).
+free, R's gradient is exact fp32 instead of bf16-rounded (:542), and all-float32 tensors are accepted (slow exact path).
 """
 import torch
 
@@ -24,17 +24,18 @@ def _dims(Q, K):
 def _check_inputs(Q, K, U, V, R):
     if Q.dim() != 4 or K.dim() != 4 or R.dim() != 4:
         raise RuntimeError("expected Q [B,H,S,d_h], K/U/V [Hkuv,E,d_e,d_h], R [B,H,S,E]")
-    expected = torch.bfloat16
-    if Q.dtype != expected or K.dtype != expected or V.dtype != expected or U.dtype != expected:
+    expected = (torch.bfloat16, torch.float32)     # float32 = the correctness instantiation (a widening over the reference)
+    if Q.dtype not in expected or K.dtype != Q.dtype or V.dtype != Q.dtype or U.dtype != Q.dtype:
         raise TypeError(
-            f"FlashMLPFunction expects all inputs in {expected}, got Q={Q.dtype}, K={K.dtype}, V={V.dtype}, U={U.dtype}")
+            f"FlashMLPFunction expects all inputs in {expected[0]} (or all in {expected[1]}), got"
+            f" Q={Q.dtype}, K={K.dtype}, V={V.dtype}, U={U.dtype}")
     if R.dtype != torch.float32:
         raise TypeError(f"R must be float32 (the router gate is computed in fp32), got {R.dtype}")
     if U.shape != K.shape or V.shape != K.shape:
         raise RuntimeError(f"K, U, V must share one shape, got {tuple(K.shape)}, {tuple(U.shape)}, {tuple(V.shape)}")
     if R.shape != (*Q.shape[:3], K.shape[1]):
         raise RuntimeError(f"R must be [B,H,S,E] = {(*Q.shape[:3], K.shape[1])}, got {tuple(R.shape)}")
-    if K.shape[2] % 32 != 0:
+    if Q.dtype == torch.bfloat16 and K.shape[2] % 32 != 0:
         raise ValueError(f"Expert dimension {K.shape[2]} must be divisible by 32")
     if not Q.is_cuda:
         raise RuntimeError("flashmhf_amd runs on the GPU only; there is no CPU path")

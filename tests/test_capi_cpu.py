@@ -39,7 +39,10 @@ def test_strerror_and_is_supported(L):
     assert L.mhffn_is_supported(64, 32, 0) == 1
     assert L.mhffn_is_supported(128, 48, 0) == 0
     assert L.mhffn_is_supported(80, 64, 0) == 0
-    assert L.mhffn_is_supported(128, 64, 1) == 0
+    assert L.mhffn_is_supported(128, 64, 1) == 1       # fp32 correctness instantiation
+    assert L.mhffn_is_supported(40, 7, 1) == 1         # ... generic in d_h (multiple of 8) and d_e
+    assert L.mhffn_is_supported(132, 64, 1) == 0
+    assert L.mhffn_is_supported(128, 64, 2) == 0
 
 
 @pytest.mark.parametrize("dims,dtype,code", [
@@ -49,7 +52,8 @@ def test_strerror_and_is_supported(L):
     ((8, 8, 3, 2048, 128, 11, 352), 0, _capi.ERR_SHAPE),
     ((0, 8, 8, 2048, 128, 11, 352), 0, _capi.ERR_SHAPE),
     ((8, 8, 8, 2048, 128, 65, 352), 0, _capi.ERR_SHAPE),
-    ((8, 8, 8, 2048, 128, 11, 352), 1, _capi.ERR_DTYPE),
+    ((8, 8, 8, 2048, 128, 11, 352), 1, 0),
+    ((8, 8, 8, 2048, 100, 11, 352), 1, _capi.ERR_HEAD_DIM),
     ((8, 8, 8, 2048, 128, 11, 352), 7, _capi.ERR_DTYPE),
 ])
 def test_check_dims_codes(L, dims, dtype, code):
@@ -81,8 +85,10 @@ def test_python_boundary_raises_reference_exception_types():
     K = torch.zeros(2, 2, 64, 128, dtype=torch.bfloat16)
     R = torch.zeros(1, 2, 8, 2)
     for mod in (FlashMLPMoE(), FlashFFNMoE()):
-        with pytest.raises(TypeError):                     # flash_mlp_moe.py:761-766
+        with pytest.raises(TypeError):                     # flash_mlp_moe.py:761-766 (mixed dtypes)
             mod(Q.float(), K, K, K, R)
+        with pytest.raises(TypeError):
+            mod(Q.half(), K.half(), K.half(), K.half(), R)
         with pytest.raises(TypeError):
             mod(Q, K, K, K, R.bfloat16())
         with pytest.raises(ValueError):                    # flash_mlp_moe.py:758-759
