@@ -1,0 +1,104 @@
+"""Size-independent properties of the HIP path at the benchmark's full 370M-layer size (B8 x S2048, H8, d_h128, E11,
+d_e352), where a CPU oracle of the whole problem would take too long, plus an oracle comparison on a token subset
+(every output row depends only on its own Q and R row) and on one batch element for the weight gradients."""
+import pytest
+import torch
+
+from oracle import mhffn_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+C2 = dict(B=8, H=8, S=2048, dh=128, E=11, de=352)
+
+
+@pytest.fixture(scope="module")
+def c2():
+    g = torch.Generator().manual_seed(1234)
+    B, H, S, dh, E, de = (C2[k] for k in ("B", "H", "S", "dh", "E", "de"))
+    Q = torch.randn(B, H, S, dh, generator=g).bfloat16()
+    K, U, V = ((torch.randn(H, E, de, dh, generator=g) * dh ** -0.5).bfloat16() for _ in range(3))
+    R = torch.sigmoid(torch.randn(B, H, S, E, generator=g) * 0.64)
+    R = R / R.sum(-1, keepdim=True)
+    dO = torch.randn(B, H, S, dh, generator=g).bfloat16()
+    return [t.to(DEV) for t in (Q, K, U, V, R, dO)]
+
+
+def test_full_size_rows_match_oracle_on_a_token_subset(c2):
+    from flashmhf_amd import mhffn_backward, mhffn_forward
+    Q, K, U, V, R, dO = c2
+    O = mhffn_forward(Q, K, U, V, R)
+    dQ, _, _, _, dR = mhffn_backward(Q, K, U, V, R, dO, grad_w_dtype=torch.float32)
+    torch.cuda.synchronize()
+    idx = torch.tensor([0, 1, 31, 32, 255, 256, 257, 1023, 1500, 2047])      # tile edges and interior
+    sub = lambda t: t[:2, :, idx].cpu()
+    ref_O = orc.mhffn_forward(sub(Q), K.cpu(), U.cpu(), V.cpu(), sub(R), compute_dtype=torch.float32)
+    ref = orc.mhffn_backward(sub(Q), K.cpu(), U.cpu(), V.cpu(), sub(R), sub(dO), compute_dtype=torch.float64)
+    for name, got, r in (("O", sub(O), ref_O), ("dQ", sub(dQ), ref[0]), ("dR", sub(dR), ref[4])):
+        m = orc.error_metrics(got.float(), r)
+        assert m["max_abs"] <= 2e-2 * max(1.0, r.abs().max().item()) and m["mean_rel"] <= 1e-2, (name, m)
+
+
+def test_full_length_weight_gradients_match_oracle_on_one_batch_element(c2):
+    from flashmhf_amd import mhffn_backward
+    Q, K, U, V, R, dO = c2
+    one = lambda t: t[:1].contiguous()
+    _, dK, dU, dV, _ = mhffn_backward(one(Q), K, U, V, one(R), one(dO), grad_w_dtype=torch.float32)
+    torch.cuda.synchronize()
+    ref = orc.mhffn_backward(one(Q).cpu(), K.cpu(), U.cpu(), V.cpu(), one(R).cpu(), one(dO).cpu(), compute_dtype=torch.float32)
+    for name, got, r in zip(("dK", "dU", "dV"), (dK, dU, dV), ref[1:4]):
+        m = orc.error_metrics(got.cpu(), r)
+        assert m["norm_max"] <= 2e-2 and m["mean_rel"] <= 1e-2, (name, m)
+
+
+def test_weight_gradients_add_over_batch_elements(c2):
+    """dK of the whole batch equals the sum of the per-batch-element dK (fp32 outputs; slices are summed in fp32)."""
+    from flashmhf_amd import mhffn_backward
+    Q, K, U, V, R, dO = c2
+    full = mhffn_backward(Q, K, U, V, R, dO, grad_w_dtype=torch.float32)[1:4]
+    parts = [torch.zeros_like(full[0]) for _ in range(3)]
+    for b in range(Q.shape[0]):
+        sl = lambda t: t[b:b + 1].contiguous()
+        g = mhffn_backward(sl(Q), K, U, V, sl(R), sl(dO), grad_w_dtype=torch.float32)[1:4]
+        for acc, x in zip(parts, g):
+            acc += x
+    torch.cuda.synchronize()
+    for name, a, b_ in zip(("dK", "dU", "dV"), full, parts):
+        err = (a - b_).abs().max().item() / a.abs().max().item()
+        assert err <= 1e-5, (name, err)
+
+
+def test_exact_symmetries_at_full_size(c2):
+    from flashmhf_amd import mhffn_forward
+    Q, K, U, V, R, _ = c2
+    O = mhffn_forward(Q, K, U, V, R)
+    # scaling the gate by a power of two commutes with every rounding step: bit-exact
+    assert torch.equal(mhffn_forward(Q, K, U, V, 2.0 * R), (2.0 * O.float()).bfloat16())
+    # tokens are independent: permuting them permutes the rows, bit for bit
+    perm = torch.randperm(Q.shape[2], device=DEV)
+    assert torch.equal(mhffn_forward(Q[:, :, perm].contiguous(), K, U, V, R[:, :, perm].contiguous()), O[:, :, perm])
+    # heads are independent
+    assert torch.equal(mhffn_forward(Q[:, 3:4].contiguous(), K[3:4].contiguous(), U[3:4].contiguous(),
+                                     V[3:4].contiguous(), R[:, 3:4].contiguous()), O[:, 3:4])
+    # a sequence cut at an odd length gives the same rows as the full one (tail masking)
+    cut = 1999
+    assert torch.equal(mhffn_forward(Q[:, :, :cut].contiguous(), K, U, V, R[:, :, :cut].contiguous()), O[:, :, :cut])
+    # zero gate -> zero output; zero K or U -> zero output
+    assert mhffn_forward(Q, K, U, V, torch.zeros_like(R)).abs().max().item() == 0
+    assert mhffn_forward(Q, torch.zeros_like(K), U, V, R).abs().max().item() == 0
+    # permuting experts jointly in (K, U, V, R) changes only the summation order
+    pe = torch.randperm(K.shape[1], device=DEV)
+    Op = mhffn_forward(Q, K[:, pe].contiguous(), U[:, pe].contiguous(), V[:, pe].contiguous(), R[..., pe].contiguous())
+    assert (Op.float() - O.float()).abs().max().item() <= 2e-2
+
+
+def test_dR_is_inner_product_of_dO_with_per_expert_output(c2):
+    from flashmhf_amd import mhffn_backward, mhffn_forward
+    Q, K, U, V, R, dO = [t[:2].contiguous() if t.dim() == 4 and t.shape[0] == 8 else t for t in c2]
+    dR = mhffn_backward(Q, K, U, V, R, dO)[4]
+    e = 5
+    onehot = torch.zeros_like(R)
+    onehot[..., e] = 1.0
+    Oe = mhffn_forward(Q, K, U, V, onehot).float()
+    ref = (Oe * dO.float()).sum(-1)
+    scale = ref.abs().max().item()
+    assert (dR[..., e] - ref).abs().max().item() <= 2e-2 * scale
