@@ -98,6 +98,9 @@ def kernel_timings(w, ins, n=10):
 # Credited GEMMs per kernel (in units of F1): the forward's three; the dQ/dR kernel's recomputed M, N, dA and the two
 # dQ products; the dK/dU/dV kernel's three output products (its own recomputation of M, N, dA is not credited).
 CREDIT = {"fwd_main": 3, "bwd_dqdr": 5, "bwd_dkdudv": 3}
+# HBM bytes per launch at workload c2 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy
+# (profiles/c2_hbm_traffic_pmc.md); counters cannot be read from inside this process, so the figures are recorded here.
+TRAFFIC_C2 = {"fwd_main": 120.6e6, "bwd_dqdr": 160.6e6, "bwd_dkdudv": 334.4e6}
 HARDWARE = {"fwd_main": 3, "bwd_dqdr": 5, "bwd_dkdudv": 6}
 
 
@@ -141,6 +144,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times (known-size reference for HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the fused MH-FFN on ONE GPU; --gpus must be 1 "
@@ -152,6 +157,13 @@ def main():
 
     from flashmhf_amd import mhffn_backward, mhffn_forward
     dev = torch.device("cuda:0")
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)           # reads 256 MiB, writes 256 MiB per launch
+        torch.cuda.synchronize()
+        del src, dst
     w = WORKLOADS[args.workload]
     ins = make_inputs(w, dev)
     Q, K, U, V, R, dO = ins
@@ -183,7 +195,7 @@ def main():
     dom = max(CREDIT, key=lambda k: kt.get(k, 0.0))
     ach = CREDIT[dom] * f1(w) / (kt[dom] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": ach / PEAK_BF16_TFLOPS, "traffic": None,
+                "frac": ach / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_C2.get(dom) if args.workload == "c2" else None,
                 "hardware_tflops": HARDWARE[dom] * f1(w) / (kt[dom] * 1e-3) / 1e12}
     kernels = {k: {"ms": v, **({"credited_tflops": CREDIT[k] * f1(w) / (v * 1e-3) / 1e12,
                                 "hardware_tflops": HARDWARE[k] * f1(w) / (v * 1e-3) / 1e12} if k in CREDIT else {})}

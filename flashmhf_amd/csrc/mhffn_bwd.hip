@@ -233,9 +233,9 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
 
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int hk = blockIdx.y, z = blockIdx.z;
+    const int hk = blockIdx.x, z = blockIdx.z;   // head index fastest: all columns of a head run on one XCD and share its L2
     const int nblk = p.E * p.nbe;
-    const int jblk = blockIdx.x * 4 + wave;
+    const int jblk = blockIdx.y * 4 + wave;
     const bool active = jblk < nblk;
     const int jb_c = active ? jblk : nblk - 1;        // idle waves of the last column recompute the last block
     const int e_w = jb_c / p.nbe;
@@ -499,7 +499,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
 
     if (active) {
         // dK^T registers 4a+b of row tile ct: c = 32ct + 8a + 4g + b, column j = l32 -> 16-byte runs along c.
-        const long wsz = (long)gridDim.y * nblk * JB * DH;   // elements of one weight tensor
+        const long wsz = (long)gridDim.x * nblk * JB * DH;   // elements of one weight tensor
         float* base = p.part + (long)z * 3 * wsz + wrow * DH;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
@@ -607,7 +607,7 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
         }
         if (d.E > 64) return hipErrorInvalidValue;   // staged R tile holds at most 64 experts
         const int nblk = d.E * nbe;
-        dim3 grid((unsigned)((nblk + 3) / 4), (unsigned)d.Hkuv, (unsigned)nslice);
+        dim3 grid((unsigned)d.Hkuv, (unsigned)((nblk + 3) / 4), (unsigned)nslice);
         if (d.S % 32 == 0)
             hipLaunchKernelGGL((mhffn_bwd_dkdudv_kernel<DH, false>), grid, dim3(256), smem, st, a);
         else
