@@ -137,6 +137,22 @@ def cpu_baseline(w, budget_s=25.0):
                       f"{med * 1e3:.1f} ms/step, tokens/s {B * S / med:.0f}"}
 
 
+def swiglu_peak_bytes(tokens, hidden, inner, device):
+    """Peak HBM beyond inputs of a SwiGLU FFN (gate/up/down nn.Linear, bf16) fwd+bwd on the same tokens: the memory
+    comparison of workload c3 (inner size from the reference's configs/baseline/configure10-TriDao-1.3B-bf16-pile.json:11)."""
+    import torch.nn.functional as F
+    x = torch.randn(tokens, hidden, device=device, dtype=torch.bfloat16, requires_grad=True)
+    gate, up = (torch.nn.Linear(hidden, inner, bias=False, device=device, dtype=torch.bfloat16) for _ in range(2))
+    down = torch.nn.Linear(inner, hidden, bias=False, device=device, dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    y = down(F.silu(gate(x)) * up(x))
+    y.backward(torch.ones_like(y))
+    torch.cuda.synchronize()
+    return int(torch.cuda.max_memory_allocated() - base)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -216,6 +232,8 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    if args.workload == "c3":
+        out["swiglu_2048_5504_peak_hbm_bytes_beyond_inputs"] = swiglu_peak_bytes(tokens, 2048, 5504, dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(out))
