@@ -102,6 +102,12 @@ __device__ __forceinline__ void mfma_result_fence(f32x16& a, f32x16& b, f32x16& 
     // are operands of the statement, so no read of them can be scheduled above it.
     asm volatile("s_nop 15\n\ts_nop 15" : "+v"(a), "+v"(b), "+v"(c));
 }
+// Never pass the same object twice to one fence: the compiler would materialise the extra operands as register copies
+// of the result, and those copies are VALU reads issued before the wait states have passed.
+__device__ __forceinline__ void mfma_result_fence(f32x16& a)
+{
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(a));
+}
 
 __device__ __forceinline__ float fast_sigmoid(float x)
 {
