@@ -221,8 +221,8 @@ struct DwArgs {
 };
 
 constexpr int DW_NST = 4;                              // LDS stages of the token-tile ring
-constexpr int DW_RTILE_B = 8 * 1024;                   // staged R tile: [E][32] fp32, E <= 64
-constexpr int DW_STAGE_B = 2 * TILE_B + DW_RTILE_B;    // Q tile | dO tile | R tile
+constexpr int DW_RTILE_B = 1024;                       // staged gate values: [4 waves][64 lanes] fp32 (each wave: its expert)
+constexpr int DW_STAGE_B = 2 * TILE_B + DW_RTILE_B;    // Q tile | dO tile | gate values
 
 template <int DH, bool TAIL>
 __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
@@ -274,7 +274,6 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     int pf_left = nt;                                 // tiles not yet requested
 
     // per-lane constants of the tile fill: this wave's two 4-row groups of the Q/dO tiles (swizzled source chunk)
-    constexpr int RINS = 8;                           // R-tile instructions per wave: covers E <= 64 with 4 waves
     int fill_row[2], fill_coff[2];
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
@@ -306,14 +305,10 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
             __builtin_amdgcn_global_load_lds((gptr_t)(qb + off), (lptr_t)(sbase + ins * 1024), 16, 0, 0);
             __builtin_amdgcn_global_load_lds((gptr_t)(gb + off), (lptr_t)(sbase + TILE_B + ins * 1024), 16, 0, 0);
         }
-        // R tile: [E][32] fp32, one 4-byte element per lane, two experts per instruction; experts past E reload the last.
+        // gate values of this wave's expert for the 32 token rows (lanes 32..63 repeat them): one 4-byte element per lane
         const int trow = TAIL ? (l32 < last ? l32 : last) : l32;
-        for (int ins = wave; 2 * ins < p.E; ins += 4) {
-            int e = 2 * ins + (lane >> 5);
-            e = e < p.E ? e : p.E - 1;
-            const unsigned off = (unsigned)((trow * p.E + e) * 4);
-            __builtin_amdgcn_global_load_lds((gptr_t)(rbp + off), (lptr_t)(sbase + 2 * TILE_B + ins * 256), 4, 0, 0);
-        }
+        __builtin_amdgcn_global_load_lds((gptr_t)(rbp + (unsigned)((trow * p.E + e_w) * 4)),
+                                         (lptr_t)(sbase + 2 * TILE_B + wave * 256), 4, 0, 0);
         // advance unless this was the last tile of the slice (then later requests reload it, harmlessly)
         const bool more = pf_left > 1;
         pf_left -= more ? 1 : 0;
@@ -328,8 +323,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     // the stage: zeroes the gate values of the rows a tail tile does not have.
     auto zero_tail = [&](int sidx, int nvalid) {
         float* sR = reinterpret_cast<float*>(smem_raw + sidx * DW_STAGE_B + 2 * TILE_B);
-        for (int ins = wave; 2 * ins < p.E; ins += 4)
-            if (l32 >= nvalid) sR[ins * 64 + lane] = 0.0f;
+        if (l32 >= nvalid) sR[wave * 64 + lane] = 0.0f;
     };
 
     const int fr = swz16(l32);
@@ -350,7 +344,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         const unsigned char* pG = pQ + TILE_B;
         // the previous tile's gate values, or zeros when there is no previous tile to contract (first step of a slice,
         // phantom steps that pad the loop): a zero gate makes P, dM and dN exactly zero
-        const float* pR = live ? reinterpret_cast<const float*>(pG + TILE_B) + e_w * 32 : sZero;
+        const float* pR = live ? reinterpret_cast<const float*>(pG + TILE_B) + wave * 64 : sZero;
 
         bf16x8 pB[2], dmB[2], dnB[2];
         bf16x8 aq[3], ag[3], vB[3];                  // operand ring: k-step ks+2 is requested while ks is consumed
@@ -366,34 +360,56 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
 #pragma unroll
         for (int a = 0; a < 4; ++a) rv[a] = *reinterpret_cast<const f32x4*>(pR + 8 * a + 4 * g);
 
-        // Element-wise work of the previous tile, one element (register index i of pm/pn/pda) at a time, in three slices
-        // of at most ~7 issue slots so that each fits under one MFMA (32 cycles): a = exp, b = sigmoid / silu,
-        // c = silu' and the three gated products.
-        float ev, sgv, slv;
-        auto ew_a = [&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            ev = __builtin_amdgcn_exp2f(-LOG2E * pm[i]);
+        // Element-wise work of the previous tile, two elements (register indices 2pr, 2pr+1 of pm/pn/pda) at a time so
+        // that no instruction waits on the one just before it, in five slices of at most six VALU instructions; one slice
+        // fits under one MFMA (32 cycles).  With sigma = 1/(1+2^(-m log2 e)), B = r sigma, A = m B (= r silu(m)):
+        //     P = A n,   dN = A dA,   dM = (B + A (1 - sigma)) (n dA)         [silu'(m) = sigma + silu(m) (1 - sigma)]
+        float ex[8][2], sg[8][2], nda[8][2], Av[8][2], Bv[8][2], s1[8][2];
+        auto slice = [&](auto pc, auto kc) {
+            constexpr int pr = decltype(pc)::value, k = decltype(kc)::value;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int i = 2 * pr + u;
+                if constexpr (k == 0) {
+                    ex[pr][u] = __builtin_amdgcn_exp2f(-LOG2E * pm[i]);
+                } else if constexpr (k == 1) {
+                    sg[pr][u] = __builtin_amdgcn_rcpf(1.0f + ex[pr][u]);
+                    nda[pr][u] = pn[i] * pda[i];
+                } else if constexpr (k == 2) {
+                    Bv[pr][u] = rv[i >> 2][i & 3] * sg[pr][u];
+                    Av[pr][u] = pm[i] * Bv[pr][u];
+                    s1[pr][u] = 1.0f - sg[pr][u];
+                } else if constexpr (k == 3) {
+                    pB[i >> 3][i & 7] = (bf16_t)(Av[pr][u] * pn[i]);
+                    dnB[i >> 3][i & 7] = (bf16_t)(Av[pr][u] * pda[i]);
+                } else {
+                    dmB[i >> 3][i & 7] = (bf16_t)(__builtin_fmaf(Av[pr][u], s1[pr][u], Bv[pr][u]) * nda[pr][u]);
+                }
+            }
         };
-        auto ew_b = [&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            sgv = __builtin_amdgcn_rcpf(1.0f + ev);
-            slv = pm[i] * sgv;                              // silu(m)
+        // Slice list 1 (24 entries, placed behind the first-product MFMAs): pairs 0..3 completely -- the s = 0 operands of
+        // the contraction -- then the exponentials of pairs 4..7.  Slice list 2 (16 entries, behind the s = 0 contraction
+        // MFMAs): the rest of pairs 4..7, which the s = 1 MFMAs need.
+        auto list1 = [&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            if constexpr (q < 20) slice(std::integral_constant<int, q / 5>{}, std::integral_constant<int, q % 5>{});
+            else slice(std::integral_constant<int, q - 16>{}, std::integral_constant<int, 0>{});
         };
-        auto ew_c = [&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            const float wv = __builtin_fmaf(slv, 1.0f - sgv, sgv);      // silu'(m)
-            const float nn = pn[i], dA = pda[i], rr = rv[i >> 2][i & 3];
-            const float rs = rr * slv;
-            pB[i >> 3][i & 7] = (bf16_t)(rs * nn);
-            dnB[i >> 3][i & 7] = (bf16_t)(rs * dA);
-            dmB[i >> 3][i & 7] = (bf16_t)((rr * wv) * (nn * dA));
+        auto list2 = [&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            slice(std::integral_constant<int, 4 + q / 4>{}, std::integral_constant<int, 1 + q % 4>{});
         };
-        auto ew_all = [&](auto ic) { ew_a(ic); ew_b(ic); ew_c(ic); };
 
-        // Phase 1: first products of this tile (24 MFMAs for d_h = 128) with elements 0..7 of the previous tile (the
-        // s = 0 operands of its contraction) dealt out between them.  One MFMA, then half an element, and so on:
-        // back-to-back MFMAs would block this wave's in-order instruction stream until the matrix pipe takes each.
-        constexpr int E1 = 8;                               // elements converted in phase 1
+        // Phase 1: first products of this tile (24 MFMAs for d_h = 128), one slice of list 1 behind each: back-to-back
+        // MFMAs would block this wave's in-order instruction stream until the matrix pipe takes each.
+        constexpr int NS1 = 3 * KS;
+        auto after_slot1 = [&](auto kc) {
+            constexpr int k = decltype(kc)::value;
+            static_for<24>([&](auto qc) {
+                if constexpr (decltype(qc)::value * NS1 / 24 == k) list1(qc);
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        };
         static_for<KS>([&](auto kc) {
             constexpr int ks = decltype(kc)::value;
             if constexpr (ks + 2 < KS) {
@@ -402,22 +418,15 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
                 ag[(ks + 2) % 3] = *reinterpret_cast<const bf16x8*>(sG + off);
                 vB[(ks + 2) % 3] = *reinterpret_cast<const bf16x8*>(sVw + off);
             }
-            constexpr int e0 = ks * E1 / KS, e1 = (ks + 1) * E1 / KS;    // element(s) of this k-step (one for KS = 8)
             if constexpr (ks == 0) mfma32_vgpr_first_bacc(m, aq[0], kB[0]);
             else mfma32_vgpr_acc_bacc(m, aq[ks % 3], kB[ks]);
-            if constexpr (e1 > e0) ew_a(std::integral_constant<int, e0>{});
-            __builtin_amdgcn_sched_barrier(0);
+            after_slot1(std::integral_constant<int, 3 * ks>{});
             if constexpr (ks == 0) mfma32_vgpr_first_bacc(n, aq[0], uB[0]);
             else mfma32_vgpr_acc_bacc(n, aq[ks % 3], uB[ks]);
-            if constexpr (e1 > e0) ew_b(std::integral_constant<int, e0>{});
-            __builtin_amdgcn_sched_barrier(0);
+            after_slot1(std::integral_constant<int, 3 * ks + 1>{});
             if constexpr (ks == 0) mfma32_vgpr_first(da, ag[0], vB[0]);
             else mfma32_vgpr_acc(da, ag[ks % 3], vB[ks % 3]);
-            if constexpr (e1 > e0) ew_c(std::integral_constant<int, e0>{});
-            static_for<(e1 - e0 > 1 ? e1 - e0 - 1 : 0)>([&](auto dc) {      // d_h < 128: more than one element per k-step
-                ew_all(std::integral_constant<int, e0 + 1 + decltype(dc)::value>{});
-            });
-            __builtin_amdgcn_sched_barrier(0);
+            after_slot1(std::integral_constant<int, 3 * ks + 2>{});
         });
 
         // Phases 2 and 3: token contraction of the previous tile, s-major.  A = Q^T / dO^T gathered from the row-major
@@ -443,19 +452,22 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
                 if constexpr (idx + 2 < NSET) request(std::integral_constant<int, idx + 2>{});
                 constexpr int ahead = (NSET - 1 - idx) < 2 ? (NSET - 1 - idx) : 2;
                 lds_tr_wait_n<4 * ahead>(tq[idx % 3], tg[idx % 3]);
-                // elements of phase 2 handled around this operand set: (16 - E1) elements over CT sets
-                constexpr int f0 = E1 + ct * (16 - E1) / CT, f1 = E1 + (ct + 1) * (16 - E1) / CT;
+                // s = 0: list 2 is dealt out over the 3 CT MFMAs of this half
+                auto after_slot2 = [&](auto kc) {
+                    constexpr int k = decltype(kc)::value;
+                    if constexpr (s == 0) {
+                        static_for<16>([&](auto qc) {
+                            if constexpr (decltype(qc)::value * (3 * CT) / 16 == k) list2(qc);
+                        });
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                };
                 dk[ct] = mfma32(tr_value(tq[idx % 3]), dmB[s], dk[ct]);
-                if constexpr (s == 0 && f1 > f0) ew_all(std::integral_constant<int, f0>{});
-                __builtin_amdgcn_sched_barrier(0);
+                after_slot2(std::integral_constant<int, 3 * ct>{});
                 du[ct] = mfma32(tr_value(tq[idx % 3]), dnB[s], du[ct]);
-                if constexpr (s == 0) {
-                    static_for<(f1 - f0 > 1 ? f1 - f0 - 1 : 0)>(
-                        [&](auto dc) { ew_all(std::integral_constant<int, f0 + 1 + decltype(dc)::value>{}); });
-                }
-                __builtin_amdgcn_sched_barrier(0);
+                after_slot2(std::integral_constant<int, 3 * ct + 1>{});
                 dv[ct] = mfma32(tr_value(tg[idx % 3]), pB[s], dv[ct]);
-                __builtin_amdgcn_sched_barrier(0);
+                after_slot2(std::integral_constant<int, 3 * ct + 2>{});
             });
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -472,6 +484,8 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     int nv0 = issue_tile(0), nv1 = issue_tile(1), nv2 = 32, nv3 = 32;   // valid rows of the tile in each stage
     auto sync_step = [&](auto st_c, int nvalid, int& nv_next) {
         constexpr int ST = decltype(st_c)::value;
+        // All of this wave's loads, not only the older tile's: the 4-byte gate loads and the 16-byte tile loads are not
+        // known to retire in issue order, so a partial count could let a load of the older tile still be in flight.
         wait_vmcnt<0>();
         if constexpr (TAIL) {
             if (nvalid < 32) zero_tail(ST, nvalid);
