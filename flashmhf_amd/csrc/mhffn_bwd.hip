@@ -269,9 +269,15 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     const int t_begin = (int)((long)ntile * z / p.nslice), t_end = (int)((long)ntile * (z + 1) / p.nslice);
     const int nt = t_end - t_begin;
 
-    // Tile cursor of the prefetcher: tile index -> (q-head of the group, batch, 32-token tile), advanced incrementally.
-    int pf_st = t_begin % nS, pf_bb = (t_begin / nS) % p.B, pf_gi = t_begin / (nS * p.B);
+    // Tile cursor of the prefetcher: tile index -> (q-head of the group, batch, 32-token tile).  It is kept as a running
+    // token-row index that advances by one of three precomputed strides (next tile of the sequence, next
+    // batch, next q-head of the group), so a step spends a handful of scalar instructions on it.
+    int pf_st = t_begin % nS, pf_bb = (t_begin / nS) % p.B;
     int pf_left = nt;                                 // tiles not yet requested
+    // (token rows are counted in 32 bits: B * H * S < 2^31 is checked on the host)
+    int pf_row = (pf_bb * p.H + hk * p.G + t_begin / (nS * p.B)) * p.S + pf_st * 32;
+    const int drow_s = p.H * p.S - (nS - 1) * 32;                              // last tile of a sequence -> next batch
+    const int drow_b = p.S - (p.B - 1) * p.H * p.S - (nS - 1) * 32;            // ... of the last batch -> next q-head
 
     // per-lane constants of the tile fill: this wave's two 4-row groups of the Q/dO tiles (swizzled source chunk)
     int fill_row[2], fill_coff[2];
@@ -291,11 +297,10 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     // and their gate value is zeroed afterwards (zero_tail), which removes them from all three products.
     // Returns the number of valid rows of the tile (32 unless it is a tail tile).
     auto issue_tile = [&](int sidx) -> int {
-        const long rb = ((long)pf_bb * p.H + hk * p.G + pf_gi) * p.S + pf_st * 32;   // first token row of the tile
         const int last = p.S - pf_st * 32 - 1;                                       // last valid row of the tile (>= 0)
-        const char* qb = reinterpret_cast<const char*>(p.Q + rb * DH);
-        const char* gb = reinterpret_cast<const char*>(p.dO + rb * DH);
-        const char* rbp = reinterpret_cast<const char*>(p.R + rb * p.E);
+        const char* qb = reinterpret_cast<const char*>(p.Q) + (long)pf_row * (DH * 2);
+        const char* gb = reinterpret_cast<const char*>(p.dO) + (long)pf_row * (DH * 2);
+        const char* rbp = reinterpret_cast<const char*>(p.R) + (long)pf_row * (p.E * 4);
         unsigned char* sbase = smem_raw + sidx * DW_STAGE_B;
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
@@ -310,13 +315,14 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         __builtin_amdgcn_global_load_lds((gptr_t)(rbp + (unsigned)((trow * p.E + e_w) * 4)),
                                          (lptr_t)(sbase + 2 * TILE_B + wave * 256), 4, 0, 0);
         // advance unless this was the last tile of the slice (then later requests reload it, harmlessly)
-        const bool more = pf_left > 1;
-        pf_left -= more ? 1 : 0;
-        const bool wrap_s = more && (pf_st + 1 == nS);
-        pf_st = more ? (wrap_s ? 0 : pf_st + 1) : pf_st;
-        const bool wrap_b = wrap_s && (pf_bb + 1 == p.B);
-        pf_bb = wrap_s ? (wrap_b ? 0 : pf_bb + 1) : pf_bb;
-        pf_gi += wrap_b ? 1 : 0;
+        // (0/1 flags and multiplies: selects here were turned into branches inside the hot loop)
+        const int more = pf_left > 1 ? 1 : 0;
+        const int ws = (pf_st + 1 == nS ? 1 : 0) * more;
+        const int wb = (pf_bb + 1 == p.B ? 1 : 0) * ws;
+        pf_left -= more;
+        pf_row += more * 32 + ws * (drow_s - 32) + wb * (drow_b - drow_s);
+        pf_st = (pf_st + more) * (1 - ws);
+        pf_bb = (pf_bb + ws) * (1 - wb);
         return last + 1;
     };
     // Called by every wave after its own loads of stage `sidx` have landed and before the barrier that publishes

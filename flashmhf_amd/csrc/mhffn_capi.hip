@@ -22,6 +22,7 @@ int check_dims_impl(const mhffn_dims* d, int dtype)
     }
     // index arithmetic inside the kernels is 64-bit for rows, 32-bit for per-(b,h) token indices and grid extents
     if ((long long)d->B > 65535 || (long long)d->S > (1ll << 30)) return MHFFN_ERR_SHAPE;
+    if ((long long)d->B * d->H * d->S >= (1ll << 31)) return MHFFN_ERR_SHAPE;   // token rows are counted in 32 bits
     return MHFFN_OK;
 }
 
