@@ -1,11 +1,11 @@
 // Fused multi-head FFN backward for gfx950 (bf16 MFMA, fp32 accumulation), two kernels:
 //
-//  (1) dQ/dR kernel -- same tiling as the forward: a workgroup owns 4 * 32*NCT tokens of one (batch, q-head) and
-//      streams the packed stage images (Kn | Un | Vn | Kt | Ut) through LDS.  Per 32-row block and wave:
-//          M^T = Kn Q^T, N^T = Un Q^T, dA^T = Vn dO^T         (recomputed, registers only)
+//  (1) dQ/dR kernel -- a workgroup of 8 waves (two per SIMD) owns 256 tokens of one (batch, q-head), 32 per wave, and
+//      streams the K, U, V blocks (32 rows at a time) through a ring of LDS stages with LDS-direct loads.  Per block:
+//          M^T = K Q^T, N^T = U Q^T, dA^T = V dO^T            (recomputed, registers only)
 //          dR_e += sum_j dA * silu(M) * N                      (fp32, before any rounding)
 //          dN^T = r_e dA^T silu(M^T),  dM^T = r_e dA^T N^T silu'(M^T)      (rounded once to bf16)
-//          dQ^T += Kt dM^T + Ut dN^T
+//          dQ^T += K^T dM^T + U^T dN^T                         (K^T, U^T: transposing reads of the same K, U tiles)
 //      Formulas: kernels/triton/flash_mlp_moe.py:401-414, :527-542.
 //
 //  (2) dK/dU/dV kernel -- a wave owns one 32-row block of K/U/V (held in registers as MFMA B operands) and loops
