@@ -20,7 +20,9 @@ ERR_NULL_POINTER, ERR_DTYPE, ERR_HEAD_DIM, ERR_EXPERT_DIM, ERR_SHAPE, ERR_WORKSP
 EXPORTS = (
     "mhffn_strerror", "mhffn_is_supported", "mhffn_check_dims", "mhffn_fwd_workspace_bytes",
     "mhffn_bwd_workspace_bytes", "mhffn_fwd", "mhffn_bwd", "mhffn_fwd_phases", "mhffn_bwd_phases",
+    "mhffn_fwd_layout", "mhffn_bwd_layout",
 )
+TOKENS_BHSD, TOKENS_BSHD = 0, 1     # layout of Q, O, dO, dQ
 FWD_PACK, FWD_MAIN, FWD_ALL = 1, 2, 3
 BWD_PACK, BWD_DQDR, BWD_DKDUDV, BWD_REDUCE, BWD_ALL = 1, 2, 4, 8, 15
 
@@ -53,6 +55,9 @@ def lib():
         L.mhffn_bwd.argtypes = [vp] * 6 + [vp] * 5 + [ctypes.c_int, vp, ctypes.c_size_t, dp, ctypes.c_int, vp]
         L.mhffn_fwd_phases.argtypes = L.mhffn_fwd.argtypes + [ctypes.c_int]
         L.mhffn_bwd_phases.argtypes = L.mhffn_bwd.argtypes + [ctypes.c_int]
+        L.mhffn_fwd_layout.argtypes = [vp] * 6 + [vp, ctypes.c_size_t, dp, ctypes.c_int, ctypes.c_int, vp, ctypes.c_int]
+        L.mhffn_bwd_layout.argtypes = ([vp] * 6 + [vp] * 5 + [ctypes.c_int, vp, ctypes.c_size_t, dp, ctypes.c_int,
+                                                              ctypes.c_int, vp, ctypes.c_int])
         _lib = L
     return _lib
 

@@ -29,6 +29,7 @@ struct DqArgs {
     bf16_t* dQ;
     float* dR;
     int H, G, S, E, nbe;
+    int tokmaj;   // Q, dO, dQ token-major ([B, S, H, d_h]) instead of [B, H, S, d_h]
 };
 
 constexpr int DQ_NST = 4;                  // LDS stages (K | U | V tiles each)
@@ -48,7 +49,8 @@ __global__ __launch_bounds__(NW * 64) void mhffn_bwd_dqdr_kernel(DqArgs p)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int h = blockIdx.x, tb = blockIdx.y, b = blockIdx.z;
     const int hk = h / p.G;
-    const long rowbase = ((long)b * p.H + h) * p.S;
+    const long rowbase = ((long)b * p.H + h) * p.S;          // rows of R, dR
+    const TokRows qrows = tok_rows(p.tokmaj, b, h, p.H, p.S);   // rows of Q, dO, dQ
     const int tok0 = tb * BT + wave * (32 * NCT);
     const int nblk = p.E * p.nbe;
     const bf16_t* Kh = p.K + (long)hk * nblk * JB * DH;
@@ -74,8 +76,8 @@ __global__ __launch_bounds__(NW * 64) void mhffn_bwd_dqdr_kernel(DqArgs p)
     for (int ct = 0; ct < NCT; ++ct) {
         int t = tok0 + ct * 32 + l32;
         t = t < p.S ? t : p.S - 1;
-        const bf16_t* qr = p.Q + (rowbase + t) * DH + 8 * g;
-        const bf16_t* gr = p.dO + (rowbase + t) * DH + 8 * g;
+        const bf16_t* qr = p.Q + (qrows.base + (long)t * qrows.stride) * DH + 8 * g;
+        const bf16_t* gr = p.dO + (qrows.base + (long)t * qrows.stride) * DH + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             q[ct][ks] = *reinterpret_cast<const bf16x8*>(qr + ks * 16);
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(NW * 64) void mhffn_bwd_dqdr_kernel(DqArgs p)
     for (int ct = 0; ct < NCT; ++ct) {
         const int t = tok0 + ct * 32 + l32;
         if (t < p.S) {
-            bf16_t* orow = p.dQ + (rowbase + t) * DH;
+            bf16_t* orow = p.dQ + (qrows.base + (long)t * qrows.stride) * DH;
 #pragma unroll
             for (int i = 0; i < CT; ++i)
 #pragma unroll
@@ -218,6 +220,7 @@ struct DwArgs {
     const float* R;
     float* part;        // [nslice][3][Hkuv][E*d_e][DH] fp32 partial sums
     int B, H, G, S, E, nbe, nslice;
+    int tokmaj;         // Q, dO token-major ([B, S, H, d_h]) instead of [B, H, S, d_h]
 };
 
 constexpr int DW_NST = 4;                              // LDS stages of the token-tile ring
@@ -246,6 +249,14 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     unsigned char* sVw = smem_raw + DW_NST * DW_STAGE_B + wave * TILE_B;
     float* sZero = reinterpret_cast<float*>(smem_raw + DW_NST * DW_STAGE_B + 4 * TILE_B);   // 32 zero gate values
     if (tid < 32) sZero[tid] = 0.0f;
+    // The first step contracts a tile that does not exist (zero gate values) out of the last stage, which no load has
+    // filled yet: clear its Q and dO tiles, or whatever bit patterns the previous kernel left there (possibly NaN or
+    // Inf as bf16) would be multiplied by those zeros.
+    {
+        u32x4 z = {0u, 0u, 0u, 0u};
+        u32x4* last_stage = reinterpret_cast<u32x4*>(smem_raw + (DW_NST - 1) * DW_STAGE_B);
+        for (int i = tid; i < 2 * TILE_B / 16; i += 256) last_stage[i] = z;
+    }
     {
         const bf16_t* vblk = p.V + (((long)hk * nblk + jb_c) * JB) * DH;
 #pragma unroll
@@ -275,9 +286,15 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     int pf_st = t_begin % nS, pf_bb = (t_begin / nS) % p.B;
     int pf_left = nt;                                 // tiles not yet requested
     // (token rows are counted in 32 bits: B * H * S < 2^31 is checked on the host)
-    int pf_row = (pf_bb * p.H + hk * p.G + t_begin / (nS * p.B)) * p.S + pf_st * 32;
+    const int pf_h0 = hk * p.G + t_begin / (nS * p.B);                        // q-head of the first tile
+    int pf_row = (pf_bb * p.H + pf_h0) * p.S + pf_st * 32;                     // row of R ([B, H, S, E])
     const int drow_s = p.H * p.S - (nS - 1) * 32;                              // last tile of a sequence -> next batch
     const int drow_b = p.S - (p.B - 1) * p.H * p.S - (nS - 1) * 32;            // ... of the last batch -> next q-head
+    // The same walk in rows of Q/dO, whose token stride is qs rows (1, or H when token-major).
+    const int qs = p.tokmaj ? p.H : 1;
+    int pf_qrow = p.tokmaj ? (pf_bb * p.S + pf_st * 32) * p.H + pf_h0 : pf_row;
+    const int dqrow_s = p.H * p.S - (nS - 1) * 32 * qs;
+    const int dqrow_b = (p.tokmaj ? 1 : p.S) - (p.B - 1) * p.H * p.S - (nS - 1) * 32 * qs;
 
     // per-lane constants of the tile fill: this wave's two 4-row groups of the Q/dO tiles (swizzled source chunk)
     int fill_row[2], fill_coff[2];
@@ -298,14 +315,14 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     // Returns the number of valid rows of the tile (32 unless it is a tail tile).
     auto issue_tile = [&](int sidx) -> int {
         const int last = p.S - pf_st * 32 - 1;                                       // last valid row of the tile (>= 0)
-        const char* qb = reinterpret_cast<const char*>(p.Q) + (long)pf_row * (DH * 2);
-        const char* gb = reinterpret_cast<const char*>(p.dO) + (long)pf_row * (DH * 2);
+        const char* qb = reinterpret_cast<const char*>(p.Q) + (long)pf_qrow * (DH * 2);
+        const char* gb = reinterpret_cast<const char*>(p.dO) + (long)pf_qrow * (DH * 2);
         const char* rbp = reinterpret_cast<const char*>(p.R) + (long)pf_row * (p.E * 4);
         unsigned char* sbase = smem_raw + sidx * DW_STAGE_B;
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
             const int row = TAIL ? (fill_row[k] < last ? fill_row[k] : last) : fill_row[k];
-            const unsigned off = (unsigned)(row * (DH * 2) + fill_coff[k]);
+            const unsigned off = (unsigned)(row * qs * (DH * 2) + fill_coff[k]);
             const int ins = wave + 4 * k;
             __builtin_amdgcn_global_load_lds((gptr_t)(qb + off), (lptr_t)(sbase + ins * 1024), 16, 0, 0);
             __builtin_amdgcn_global_load_lds((gptr_t)(gb + off), (lptr_t)(sbase + TILE_B + ins * 1024), 16, 0, 0);
@@ -321,6 +338,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         const int wb = (pf_bb + 1 == p.B ? 1 : 0) * ws;
         pf_left -= more;
         pf_row += more * 32 + ws * (drow_s - 32) + wb * (drow_b - drow_s);
+        pf_qrow += more * 32 * qs + ws * (dqrow_s - 32 * qs) + wb * (dqrow_b - dqrow_s);
         pf_st = (pf_st + more) * (1 - ws);
         pf_bb = (pf_bb + ws) * (1 - wb);
         return last + 1;
@@ -490,8 +508,8 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     int nv0 = issue_tile(0), nv1 = issue_tile(1), nv2 = 32, nv3 = 32;   // valid rows of the tile in each stage
     auto sync_step = [&](auto st_c, int nvalid, int& nv_next) {
         constexpr int ST = decltype(st_c)::value;
-        // All of this wave's loads, not only the older tile's: the 4-byte gate loads and the 16-byte tile loads are not
-        // known to retire in issue order, so a partial count could let a load of the older tile still be in flight.
+        // All of this wave's loads, not only the older tile's: a partial count (the next tile's loads still in flight)
+        // measured no faster.
         wait_vmcnt<0>();
         if constexpr (TAIL) {
             if (nvalid < 32) zero_tail(ST, nvalid);
@@ -594,7 +612,7 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
 
     if (phases & 2) {
         DqArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R,
-                 (bf16_t*)dQ, dR, d.H, G, d.S, d.E, nbe};
+                 (bf16_t*)dQ, dR, d.H, G, d.S, d.E, nbe, d.tokmaj};
         const int tokw = NW * 32 * NCT;
         const int smem = DQ_NST * DQ_STAGE_B + d.E * tokw * (int)sizeof(float);
         if (smem > 160 * 1024) return hipErrorInvalidValue;
@@ -613,7 +631,7 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
     const int nslice = pick_nslice(d);
     if (phases & 4) {
         DwArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, part,
-                 d.B, d.H, G, d.S, d.E, nbe, nslice};
+                 d.B, d.H, G, d.S, d.E, nbe, nslice, d.tokmaj};
         const int smem = DW_NST * DW_STAGE_B + 4 * TILE_B + 128;
         static bool attr_done = false;   // dynamic LDS above 64 KB must be opted into, per kernel
         if (!attr_done) {

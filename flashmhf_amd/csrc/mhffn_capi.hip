@@ -26,7 +26,10 @@ int check_dims_impl(const mhffn_dims* d, int dtype)
     return MHFFN_OK;
 }
 
-mhffn::Dims to_dims(const mhffn_dims* d) { return mhffn::Dims{d->B, d->H, d->Hkuv, d->S, d->d_h, d->E, d->d_e}; }
+mhffn::Dims to_dims(const mhffn_dims* d, int token_layout = 0)
+{
+    return mhffn::Dims{d->B, d->H, d->Hkuv, d->S, d->d_h, d->E, d->d_e, token_layout};
+}
 
 }  // namespace
 
@@ -71,17 +74,18 @@ size_t mhffn_bwd_workspace_bytes(const mhffn_dims* dims, int dtype)
     return mhffn::bwd_workspace_bytes_bf16(to_dims(dims));
 }
 
-int mhffn_fwd_phases(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
-                     void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream,
-                     int phases)
+int mhffn_fwd_layout(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
+                     void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, int token_layout,
+                     void* stream, int phases)
 {
     const int rc = check_dims_impl(dims, dtype);
     if (rc != MHFFN_OK) return rc;
+    if (token_layout != MHFFN_TOKENS_BHSD && token_layout != MHFFN_TOKENS_BSHD) return MHFFN_ERR_SHAPE;
     if (!Q || !K || !U || !V || !R || !O) return MHFFN_ERR_NULL_POINTER;
     if (!aligned16(Q) || !aligned16(K) || !aligned16(U) || !aligned16(V) || !aligned16(R) || !aligned16(O) ||
         !aligned16(workspace))
         return MHFFN_ERR_ALIGNMENT;
-    const mhffn::Dims d = to_dims(dims);
+    const mhffn::Dims d = to_dims(dims, token_layout);
     if (dtype == MHFFN_DTYPE_F32) {
         if (!(phases & MHFFN_FWD_MAIN)) return MHFFN_OK;
         return mhffn::launch_fwd_f32(Q, K, U, V, R, O, d, (hipStream_t)stream) == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
@@ -92,25 +96,33 @@ int mhffn_fwd_phases(const void* Q, const void* K, const void* U, const void* V,
     return err == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
 }
 
+int mhffn_fwd_phases(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
+                     void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream,
+                     int phases)
+{
+    return mhffn_fwd_layout(Q, K, U, V, R, O, workspace, workspace_bytes, dims, dtype, MHFFN_TOKENS_BHSD, stream, phases);
+}
+
 int mhffn_fwd(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
               void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream)
 {
     return mhffn_fwd_phases(Q, K, U, V, R, O, workspace, workspace_bytes, dims, dtype, stream, MHFFN_FWD_ALL);
 }
 
-int mhffn_bwd_phases(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
+int mhffn_bwd_layout(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
                      void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_dtype,
-                     void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream,
-                     int phases)
+                     void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, int token_layout,
+                     void* stream, int phases)
 {
     const int rc = check_dims_impl(dims, dtype);
     if (rc != MHFFN_OK) return rc;
+    if (token_layout != MHFFN_TOKENS_BHSD && token_layout != MHFFN_TOKENS_BSHD) return MHFFN_ERR_SHAPE;
     if (grad_w_dtype != MHFFN_DTYPE_BF16 && grad_w_dtype != MHFFN_DTYPE_F32) return MHFFN_ERR_DTYPE;
     if (!Q || !K || !U || !V || !R || !dO || !dQ || !dK || !dU || !dV || !dR) return MHFFN_ERR_NULL_POINTER;
     const void* ptrs[] = {Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, workspace};
     for (const void* p : ptrs)
         if (!aligned16(p)) return MHFFN_ERR_ALIGNMENT;
-    const mhffn::Dims d = to_dims(dims);
+    const mhffn::Dims d = to_dims(dims, token_layout);
     const size_t need = dtype == MHFFN_DTYPE_F32 ? mhffn::bwd_workspace_bytes_f32(d) : mhffn::bwd_workspace_bytes_bf16(d);
     if (need > 0 && (!workspace || workspace_bytes < need)) return MHFFN_ERR_WORKSPACE;
     if (dtype == MHFFN_DTYPE_F32)
@@ -122,6 +134,15 @@ int mhffn_bwd_phases(const void* Q, const void* K, const void* U, const void* V,
                                                   grad_w_dtype == MHFFN_DTYPE_F32, workspace, d, (hipStream_t)stream,
                                                   phases);
     return err == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
+}
+
+int mhffn_bwd_phases(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
+                     void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_dtype,
+                     void* workspace, size_t workspace_bytes, const mhffn_dims* dims, int dtype, void* stream,
+                     int phases)
+{
+    return mhffn_bwd_layout(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_dtype, workspace, workspace_bytes, dims, dtype,
+                            MHFFN_TOKENS_BHSD, stream, phases);
 }
 
 int mhffn_bwd(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,

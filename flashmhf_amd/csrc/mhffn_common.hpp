@@ -241,7 +241,18 @@ __device__ __forceinline__ void wait_vmcnt()
 // Host-side launch entry points (defined in the per-kernel .hip files).
 struct Dims {
     int B, H, Hkuv, S, d_h, E, d_e;
+    int tokmaj;   // layout of Q, O, dO, dQ: 0 = [B, H, S, d_h], 1 = [B, S, H, d_h] (token-major, heads interleaved)
 };
+
+// Rows (units of d_h elements) of Q/O/dO/dQ: token t of (batch b, q-head h) is row base + t * stride.
+struct TokRows {
+    long base;
+    int stride;
+};
+__host__ __device__ inline TokRows tok_rows(int tokmaj, int b, int h, int H, int S)
+{
+    return tokmaj ? TokRows{(long)b * S * H + h, H} : TokRows{((long)b * H + h) * S, 1};
+}
 
 size_t fwd_workspace_bytes_bf16(const Dims& d);
 size_t bwd_workspace_bytes_bf16(const Dims& d);

@@ -22,17 +22,19 @@ struct F32Args {
     const float *Q, *K, *U, *V, *R, *dO;
     float *O, *dQ, *dR, *part;
     int B, H, G, S, DH, E, DE, nslice;
+    int tokmaj;   // Q, O, dO, dQ token-major ([B, S, H, d_h]) instead of [B, H, S, d_h]
 };
 
 __device__ __forceinline__ float sigmoid_exact(float x) { return 1.0f / (1.0f + __expf(-x)); }
 
-// Loads a [rows x DH] fp32 tile (row stride DH in global) into LDS with row stride DH + 1; rows >= valid are zeroed.
-__device__ __forceinline__ void load_tile(float* dst, const float* src, int valid, int DH, int tid)
+// Loads a [rows x DH] fp32 tile (row stride `rs` rows of DH elements in global) into LDS with row stride DH + 1; rows >=
+// valid are zeroed.
+__device__ __forceinline__ void load_tile(float* dst, const float* src, int valid, int DH, int tid, int rs = 1)
 {
     const int LD = DH + 1;
     for (int i = tid; i < 32 * DH; i += 256) {
         const int r = i / DH, c = i % DH;
-        dst[r * LD + c] = r < valid ? src[(long)r * DH + c] : 0.0f;
+        dst[r * LD + c] = r < valid ? src[(long)r * rs * DH + c] : 0.0f;
     }
 }
 
@@ -47,9 +49,11 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(F32Args p)
     float* sA = sV + 32 * LD;          // [TT][JC + 1]
     const int tid = threadIdx.x, t = tid >> 3, jl = tid & 7, cg = tid & 7;
     const int h = blockIdx.x, tb = blockIdx.y, b = blockIdx.z, hk = h / p.G;
-    const long rowbase = ((long)b * p.H + h) * p.S + (long)tb * TT;
+    const long rowbase = ((long)b * p.H + h) * p.S + (long)tb * TT;   // rows of R
+    const TokRows qr = tok_rows(p.tokmaj, b, h, p.H, p.S);
+    const long qrow0 = qr.base + (long)tb * TT * qr.stride;           // rows of Q, O
     const int tvalid = min(TT, p.S - tb * TT);
-    load_tile(sQ, p.Q + rowbase * DH, tvalid, DH, tid);
+    load_tile(sQ, p.Q + qrow0 * DH, tvalid, DH, tid, qr.stride);
 
     float acc[MAXC];
 #pragma unroll
@@ -87,7 +91,7 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(F32Args p)
     if (t < tvalid)
 #pragma unroll
         for (int i = 0; i < MAXC; ++i)
-            if (i < NC) p.O[(rowbase + t) * DH + cg + 8 * i] = acc[i];
+            if (i < NC) p.O[(qrow0 + (long)t * qr.stride) * DH + cg + 8 * i] = acc[i];
 }
 
 __global__ __launch_bounds__(256) void dqdr_f32_kernel(F32Args p)
@@ -104,10 +108,12 @@ __global__ __launch_bounds__(256) void dqdr_f32_kernel(F32Args p)
     float* sDR = sDN + TT * (JC + 1);   // [TT][8] per-thread partials of dR
     const int tid = threadIdx.x, t = tid >> 3, jl = tid & 7, cg = tid & 7;
     const int h = blockIdx.x, tb = blockIdx.y, b = blockIdx.z, hk = h / p.G;
-    const long rowbase = ((long)b * p.H + h) * p.S + (long)tb * TT;
+    const long rowbase = ((long)b * p.H + h) * p.S + (long)tb * TT;   // rows of R, dR
+    const TokRows qr = tok_rows(p.tokmaj, b, h, p.H, p.S);
+    const long qrow0 = qr.base + (long)tb * TT * qr.stride;           // rows of Q, dO, dQ
     const int tvalid = min(TT, p.S - tb * TT);
-    load_tile(sQ, p.Q + rowbase * DH, tvalid, DH, tid);
-    load_tile(sG, p.dO + rowbase * DH, tvalid, DH, tid);
+    load_tile(sQ, p.Q + qrow0 * DH, tvalid, DH, tid, qr.stride);
+    load_tile(sG, p.dO + qrow0 * DH, tvalid, DH, tid, qr.stride);
 
     float acc[MAXC];
 #pragma unroll
@@ -158,7 +164,7 @@ __global__ __launch_bounds__(256) void dqdr_f32_kernel(F32Args p)
     if (t < tvalid)
 #pragma unroll
         for (int i = 0; i < MAXC; ++i)
-            if (i < NC) p.dQ[(rowbase + t) * DH + cg + 8 * i] = acc[i];
+            if (i < NC) p.dQ[(qrow0 + (long)t * qr.stride) * DH + cg + 8 * i] = acc[i];
 }
 
 // One workgroup owns a 32-row chunk of K/U/V of one kuv-head and a slice of the token tiles; partial sums go to
@@ -195,8 +201,10 @@ __global__ __launch_bounds__(256) void dkdudv_f32_kernel(F32Args p)
         const long rowbase = ((long)bb * p.H + hk * p.G + gi) * p.S + (long)st * TT;
         const int tvalid = min(TT, p.S - st * TT);
         __syncthreads();
-        load_tile(sQ, p.Q + rowbase * DH, tvalid, DH, tid);
-        load_tile(sG, p.dO + rowbase * DH, tvalid, DH, tid);
+        const TokRows qr = tok_rows(p.tokmaj, bb, hk * p.G + gi, p.H, p.S);
+        const long qrow0 = qr.base + (long)st * TT * qr.stride;
+        load_tile(sQ, p.Q + qrow0 * DH, tvalid, DH, tid, qr.stride);
+        load_tile(sG, p.dO + qrow0 * DH, tvalid, DH, tid, qr.stride);
         __syncthreads();
         const float r = t < tvalid ? p.R[(rowbase + t) * p.E + e] : 0.0f;
 #pragma unroll
@@ -278,7 +286,7 @@ hipError_t launch_fwd_f32(const void* Q, const void* K, const void* U, const voi
     F32Args a{};
     a.Q = (const float*)Q; a.K = (const float*)K; a.U = (const float*)U; a.V = (const float*)V; a.R = R;
     a.O = (float*)O;
-    a.B = d.B; a.H = d.H; a.G = d.H / d.Hkuv; a.S = d.S; a.DH = d.d_h; a.E = d.E; a.DE = d.d_e;
+    a.B = d.B; a.H = d.H; a.G = d.H / d.Hkuv; a.S = d.S; a.DH = d.d_h; a.E = d.E; a.DE = d.d_e; a.tokmaj = d.tokmaj;
     const int smem = (4 * 32 * (d.d_h + 1) + TT * (JC + 1)) * (int)sizeof(float);
     static bool attr_done = false;
     if (!attr_done) {
@@ -299,7 +307,7 @@ hipError_t launch_bwd_f32(const void* Q, const void* K, const void* U, const voi
     F32Args a{};
     a.Q = (const float*)Q; a.K = (const float*)K; a.U = (const float*)U; a.V = (const float*)V; a.R = R;
     a.dO = (const float*)dO; a.dQ = (float*)dQ; a.dR = dR; a.part = (float*)ws;
-    a.B = d.B; a.H = d.H; a.G = d.H / d.Hkuv; a.S = d.S; a.DH = d.d_h; a.E = d.E; a.DE = d.d_e;
+    a.B = d.B; a.H = d.H; a.G = d.H / d.Hkuv; a.S = d.S; a.DH = d.d_h; a.E = d.E; a.DE = d.d_e; a.tokmaj = d.tokmaj;
     a.nslice = f32_nslice(d);
     static bool attr_done = false;
     if (!attr_done) {

@@ -30,6 +30,7 @@ struct FwdArgs {
     const float* R;
     bf16_t* O;
     int H, G, S, E, nbe;  // G = H / Hkuv, nbe = d_e / 32 blocks per expert
+    int tokmaj;           // Q, O token-major ([B, S, H, d_h]) instead of [B, H, S, d_h]
 };
 
 constexpr int FWD_NST = 4;                 // LDS stages (K | U | V tiles each)
@@ -48,7 +49,8 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int h = blockIdx.x, tb = blockIdx.y, b = blockIdx.z;
     const int hk = h / p.G;
-    const long rowbase = ((long)b * p.H + h) * p.S;
+    const long rowbase = ((long)b * p.H + h) * p.S;          // rows of R
+    const TokRows qrows = tok_rows(p.tokmaj, b, h, p.H, p.S);   // rows of Q and O
     const int tok0 = tb * BT + wave * 64;
     const int nblk = p.E * p.nbe;
     const long wbase = (long)hk * nblk * JB * DH;
@@ -76,7 +78,7 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     for (int ct = 0; ct < 2; ++ct) {
         int t = tok0 + ct * 32 + l32;
         t = t < p.S ? t : p.S - 1;
-        const bf16_t* qr = p.Q + (rowbase + t) * DH + 8 * g;
+        const bf16_t* qr = p.Q + (qrows.base + (long)t * qrows.stride) * DH + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) q[ct][ks] = *reinterpret_cast<const bf16x8*>(qr + ks * 16);
     }
@@ -212,7 +214,7 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     for (int ct = 0; ct < 2; ++ct) {
         const int t = tok0 + ct * 32 + l32;
         if (t < p.S) {
-            bf16_t* orow = p.O + (rowbase + t) * DH;
+            bf16_t* orow = p.O + (qrows.base + (long)t * qrows.stride) * DH;
 #pragma unroll
             for (int i = 0; i < CT; ++i)
 #pragma unroll
@@ -252,7 +254,8 @@ hipError_t launch_fwd_bf16(const void* Q, const void* K, const void* U, const vo
     (void)ws;
     if (!(phases & 2)) return hipSuccess;
     FwdArgs a{(const bf16_t*)Q, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, (bf16_t*)O,
-              d.H,              d.H / d.Hkuv,     d.S,              d.E,              d.d_e / JB};
+              d.H,              d.H / d.Hkuv,     d.S,              d.E,              d.d_e / JB,
+              d.tokmaj};
     switch (d.d_h) {
         case 64: return launch_fwd_t<64>(a, d, st);
         case 96: return launch_fwd_t<96>(a, d, st);

@@ -18,7 +18,7 @@ class FlashFFNMoEFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         Q, K, U, V, R = ctx.saved_tensors
-        dQ, dK, dU, dV, dR = mhffn_backward(Q, K, U, V, R, grad_output.contiguous(), grad_w_dtype=torch.float32)
+        dQ, dK, dU, dV, dR = mhffn_backward(Q, K, U, V, R, grad_output, grad_w_dtype=torch.float32)
         return dQ.float(), dK, dU, dV, dR
 
 

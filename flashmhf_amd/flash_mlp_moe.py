@@ -7,6 +7,11 @@
 Same call signature, tensor contract, saved tensors (Q, K, U, V, R only -- no activations) and exception types.
 Differences, all widening: d_e may be any multiple of 32 (the reference needs 64, :758), the sequence length is
 free, R's gradient is exact fp32 instead of bf16-rounded (:542), and all-float32 tensors are accepted (slow exact path).
+
+Q may also be the transposed view of a contiguous [B,S,H,d_h] tensor -- what ``w_self(x).view(B,S,H,d_h).transpose(1,2)``
+is before the caller's ``.contiguous()`` (models/flashmhf/modeling_mhffnmoe.py:362,374).  The kernels then read it in place
+and O (and dQ) come back in the same token-major layout, so ``O.transpose(1,2).contiguous().view(B,S,hid)`` (:408) copies
+nothing.
 """
 import torch
 
@@ -44,6 +49,22 @@ def _check_inputs(Q, K, U, V, R):
             raise RuntimeError(f"{name} is on {t.device}, Q on {Q.device}")
 
 
+def _token_layout(Q):
+    """(layout code, tensor to pass): [B,H,S,d_h] contiguous, or the transposed view of a contiguous [B,S,H,d_h]."""
+    if Q.is_contiguous():
+        return _capi.TOKENS_BHSD, Q
+    if Q.transpose(1, 2).is_contiguous():
+        return _capi.TOKENS_BSHD, Q
+    return _capi.TOKENS_BHSD, Q.contiguous()
+
+
+def _as_layout(t, layout):
+    """`t` ([B,H,S,d_h] logical shape) with the memory layout `layout`, copying only if it has another one."""
+    if layout == _capi.TOKENS_BSHD:
+        return t if t.transpose(1, 2).is_contiguous() else t.transpose(1, 2).contiguous().transpose(1, 2)
+    return t.contiguous()
+
+
 def _ws(nbytes, device):
     return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)
 
@@ -51,17 +72,19 @@ def _ws(nbytes, device):
 def mhffn_forward(Q, K, U, V, R):
     """Launches the fused forward on the current stream and returns O (same shape and dtype as Q)."""
     _check_inputs(Q, K, U, V, R)
-    Q, K, U, V, R = (t.contiguous() for t in (Q, K, U, V, R))
+    layout, Q = _token_layout(Q)
+    K, U, V, R = (t.contiguous() for t in (K, U, V, R))
     L = _capi.lib()
     dims = _dims(Q, K)
     code = _capi.torch_dtype_code(Q.dtype)
     _capi.raise_for_code(L.mhffn_check_dims(dims, code), "mhffn_fwd")
-    O = torch.empty_like(Q)
+    O = torch.empty_strided(Q.shape, Q.stride(), dtype=Q.dtype, device=Q.device)
     nbytes = L.mhffn_fwd_workspace_bytes(dims, code)
     ws = _ws(nbytes, Q.device)
     with torch.cuda.device(Q.device):
-        rc = L.mhffn_fwd(Q.data_ptr(), K.data_ptr(), U.data_ptr(), V.data_ptr(), R.data_ptr(), O.data_ptr(),
-                         ws.data_ptr(), ws.numel(), dims, code, torch.cuda.current_stream().cuda_stream)
+        rc = L.mhffn_fwd_layout(Q.data_ptr(), K.data_ptr(), U.data_ptr(), V.data_ptr(), R.data_ptr(), O.data_ptr(),
+                                ws.data_ptr(), ws.numel(), dims, code, layout,
+                                torch.cuda.current_stream().cuda_stream, _capi.FWD_ALL)
     _capi.raise_for_code(rc, "mhffn_fwd")
     return O
 
@@ -71,21 +94,22 @@ def mhffn_backward(Q, K, U, V, R, dO, grad_w_dtype=torch.bfloat16):
     dK/dU/dV have ``grad_w_dtype`` (bf16 as flash_mlp_moe.py:808-810, or fp32 as flash_ffn_moe_torch.py:18-20)."""
     _check_inputs(Q, K, U, V, R)
     assert dO.shape == Q.shape, "grad_output shape should be the same as Q"
-    Q, K, U, V, R = (t.contiguous() for t in (Q, K, U, V, R))
-    dO = dO.to(Q.dtype).contiguous()
+    layout, Q = _token_layout(Q)
+    K, U, V, R = (t.contiguous() for t in (K, U, V, R))
+    dO = _as_layout(dO.to(Q.dtype), layout)
     L = _capi.lib()
     dims = _dims(Q, K)
     code = _capi.torch_dtype_code(Q.dtype)
     _capi.raise_for_code(L.mhffn_check_dims(dims, code), "mhffn_bwd")
-    dQ = torch.empty_like(Q)
+    dQ = torch.empty_strided(Q.shape, Q.stride(), dtype=Q.dtype, device=Q.device)
     dK, dU, dV = (torch.empty(K.shape, dtype=grad_w_dtype, device=K.device) for _ in range(3))
     dR = torch.empty_like(R)
     ws = _ws(L.mhffn_bwd_workspace_bytes(dims, code), Q.device)
     with torch.cuda.device(Q.device):
-        rc = L.mhffn_bwd(Q.data_ptr(), K.data_ptr(), U.data_ptr(), V.data_ptr(), R.data_ptr(), dO.data_ptr(),
-                         dQ.data_ptr(), dK.data_ptr(), dU.data_ptr(), dV.data_ptr(), dR.data_ptr(),
-                         _capi.torch_dtype_code(grad_w_dtype), ws.data_ptr(), ws.numel(), dims, code,
-                         torch.cuda.current_stream().cuda_stream)
+        rc = L.mhffn_bwd_layout(Q.data_ptr(), K.data_ptr(), U.data_ptr(), V.data_ptr(), R.data_ptr(), dO.data_ptr(),
+                                dQ.data_ptr(), dK.data_ptr(), dU.data_ptr(), dV.data_ptr(), dR.data_ptr(),
+                                _capi.torch_dtype_code(grad_w_dtype), ws.data_ptr(), ws.numel(), dims, code, layout,
+                                torch.cuda.current_stream().cuda_stream, _capi.BWD_ALL)
     _capi.raise_for_code(rc, "mhffn_bwd")
     return dQ, dK, dU, dV, dR
 

@@ -111,6 +111,26 @@ int mhffn_bwd_phases(const void* Q, const void* K, const void* U, const void* V,
                      void* workspace, size_t workspace_bytes,
                      const mhffn_dims* dims, int dtype, void* stream, int phases);
 
+/* Token-major variants: Q, O, dO, dQ are [B, S, H, d_h] (MHFFN_TOKENS_BSHD) -- the layout the caller's projections
+ * produce and consume -- instead of [B, H, S, d_h] (MHFFN_TOKENS_BHSD, what the calls above use).  K, U, V, R, dR and all
+ * other conventions are unchanged; results are identical to the [B, H, S, d_h] calls on the transposed tensors.
+ * With them the caller drops the two transposes-with-copy around the operator
+ * (models/flashmhf/modeling_mhffnmoe.py:374 `Q_multihead.transpose(1, 2).contiguous()` and
+ * :408 `.transpose(1, 2).contiguous().view(batch_size, seq_len, hidden_size)`).  `phases` as in the *_phases calls. */
+enum {
+    MHFFN_TOKENS_BHSD = 0,
+    MHFFN_TOKENS_BSHD = 1
+};
+int mhffn_fwd_layout(const void* Q, const void* K, const void* U, const void* V, const float* R,
+                     void* O, void* workspace, size_t workspace_bytes,
+                     const mhffn_dims* dims, int dtype, int token_layout, void* stream, int phases);
+int mhffn_bwd_layout(const void* Q, const void* K, const void* U, const void* V, const float* R,
+                     const void* dO,
+                     void* dQ, void* dK, void* dU, void* dV, float* dR,
+                     int grad_w_dtype,
+                     void* workspace, size_t workspace_bytes,
+                     const mhffn_dims* dims, int dtype, int token_layout, void* stream, int phases);
+
 #ifdef __cplusplus
 }
 #endif
