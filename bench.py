@@ -1,12 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the fused multi-head FFN hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3|c4] [--no-cpu]
 
 One "step" = one forward + one backward of the fused operator (through the C ABI, on torch's current stream) over
 one synthetic batch already resident in HBM.  Prints ONE JSON line.  Credited FLOPs: F1 = 2*T*H*E*d_e*d_h per
 GEMM; forward 3*F1, backward 8*F1 (recompute M,N + dA + 2 dQ + dK + dU + dV), fwd+bwd 11*F1 -- recomputation beyond
 that (the two-kernel backward runs 11*F1 on the hardware, 14*F1 with the forward) is not credited.
+
+Workload c4 is different in kind: one forward + backward of a whole random-init decoder (20 blocks of causal attention +
+the MH-FFN block of workload c3's shape, vocabulary 50,304) on batch 2 x 4096 random token ids; it reports tokens/s and
+peak memory only.
 """
 import argparse
 import json
@@ -27,6 +31,9 @@ WORKLOADS = {
     "c2": dict(B=8, S=2048, H=8, d_h=128, E=11, d_e=352, passes="fwd+bwd",
                label="370M layer fwd+bwd, bf16, B8xS2048=16384 tokens, H8 d_h128 E11 d_e352"),
     "c3": dict(B=4, S=8192, H=16, d_h=128, E=22, d_e=352, passes="fwd+bwd", label="1.3B layer fwd+bwd, bf16, 32768 tokens"),
+    "c4": dict(B=2, S=4096, H=16, d_h=128, E=22, d_e=352, layers=20, vocab=50304, attn_heads=16, passes="model",
+               label="1.3B decoder (20 blocks: causal MHA + MH-FFN H16 d_h128 E22 d_e352, RMSNorm, vocab 50304), "
+                     "one bf16 forward+backward, B2xS4096 random token ids"),
 }
 
 
@@ -153,6 +160,49 @@ def swiglu_peak_bytes(tokens, hidden, inner, device):
     return int(torch.cuda.max_memory_allocated() - base)
 
 
+def bench_model(w, args, dev):
+    """Workload c4: one training step (forward + backward) of the whole decoder; tokens/s and peak memory."""
+    from flashmhf_amd import MHFFNDecoder
+    torch.manual_seed(0)
+    hid = w["H"] * w["d_h"]
+    with torch.device(dev):
+        model = MHFFNDecoder(w["vocab"], hid, w["layers"], w["attn_heads"], w["H"], w["E"], w["d_e"],
+                             apply_rmsnorm=True).to(torch.bfloat16)
+    n_params = sum(p.numel() for p in model.parameters())
+    ids = torch.randint(0, w["vocab"], (w["B"], w["S"]), device=dev, generator=torch.Generator(dev).manual_seed(0))
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        loss = model(ids, labels=ids)
+        loss.backward()
+        return loss
+
+    for _ in range(args.warmup):
+        loss = step()
+    torch.cuda.synchronize()
+    base_mem = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    tokens = w["B"] * w["S"]
+    ffn_flops = w["layers"] * 11 * f1(w)
+    out = {
+        "metric": "1.3B decoder forward+backward tokens/s + peak memory, 1 GPU", "value": tokens / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"c4: {w['label']}", "parameters": n_params},
+        "loss": float(loss.detach()),
+        "peak_memory_bytes": {"max_allocated": int(torch.cuda.max_memory_allocated()),
+                              "parameters_and_grads_before_step": int(base_mem)},
+        "fused_ffn_credited_tflops_if_it_were_the_whole_step": ffn_flops / (ms * 1e-3) / 1e12,
+        "roofline": None, "cpu_baseline": None,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -181,6 +231,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     w = WORKLOADS[args.workload]
+    if w["passes"] == "model":
+        return bench_model(w, args, dev)
     ins = make_inputs(w, dev)
     Q, K, U, V, R, dO = ins
     bwd = "bwd" in w["passes"]

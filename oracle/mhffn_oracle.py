@@ -156,3 +156,28 @@ def error_metrics(x, ref):
         "norm_max": (d.max() / ref.abs().max().clamp(min=1e-30)).item(),
         "mean_rel": (d.sum() / ref.abs().sum().clamp(min=1e-30)).item(),
     }
+
+
+def mhffn_block_forward(x, w_self, w_self_2, K, U, V, *, num_heads, router=None, w_router=None, q_norm_weight=None,
+                        eps=1e-6, compute_dtype=torch.float32):
+    """One MH-FFN block as the reference module computes it (models/flashmhf/modeling_mhffnmoe.py:352-431, eager
+    branch), differentiable in every argument: Q = x w_self^T split into heads, optional per-head RMSNorm in fp32
+    (:97-135), gate from the per-head Q through ``router`` [H,d_h,E] (:384-386) or, if ``w_router`` [hid, H*E] is given,
+    from x; the eager expert loop; heads merged; w_self_2.  Linear weights are [out, in] as nn.Linear stores them."""
+    B, S, hid = x.shape
+    H = num_heads
+    E = K.shape[1]
+    xc = x.to(compute_dtype)
+    q = (xc @ w_self.to(compute_dtype).t()).view(B, S, H, hid // H)
+    if q_norm_weight is not None:
+        qf = q.float()
+        q = (qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps) * q_norm_weight.float()).to(compute_dtype)
+    Qh = q.transpose(1, 2)
+    if w_router is not None:
+        logits = (x.float() @ w_router.float()).view(B, S, H, E).transpose(1, 2)
+    else:
+        logits = Qh.float() @ router.float()
+    Rs = logits.sigmoid()
+    R = Rs / Rs.sum(-1, keepdim=True).clamp(min=1e-20)
+    Oh = mhffn_forward(Qh, K, U, V, R, compute_dtype=compute_dtype)
+    return Oh.transpose(1, 2).reshape(B, S, hid) @ w_self_2.to(compute_dtype).t()
