@@ -4,3 +4,4 @@ reference's operator boundary.  See ``flash_mlp_moe`` (Triton-path signature) an
 from .flash_mlp_moe import FlashMLPFunction, FlashMLPMoE, mhffn_backward, mhffn_forward  # noqa: F401
 from .flash_ffn_moe_torch import FlashFFNMoE, FlashFFNMoEFunction  # noqa: F401
 from .mhffn_layer import MHFFNDecoder, MHFFNLayer  # noqa: F401
+from .flash_mlp import FlashMLP  # noqa: F401

@@ -107,6 +107,24 @@ def test_python_boundary_raises_reference_exception_types():
             mod(Q, K, K, K, R[..., :1])
 
 
+def test_legacy_single_expert_signature_checks():
+    """flash_mlp.py:1050-1058: only SiLU, no dot scaling, U required -- all ValueError, before any GPU work."""
+    from flashmhf_amd import FlashMLP
+    Q = torch.zeros(1, 2, 8, 64, dtype=torch.bfloat16)
+    W = torch.zeros(2, 32, 64, dtype=torch.bfloat16)
+    op = FlashMLP()
+    with pytest.raises(ValueError):
+        op(Q, W, W, W, False, 1.0, 1.0, "gelu")
+    with pytest.raises(ValueError):
+        op(Q, W, W, W, True, 1.0, 1.0, "silu")
+    with pytest.raises(ValueError):
+        op(Q, W, W, W, False, 2.0, 1.0, "silu")
+    with pytest.raises(ValueError):
+        op(Q, W, None, W, False, 1.0, 1.0, "silu")
+    with pytest.raises(RuntimeError):          # CPU tensors: there is no CPU path
+        op(Q, W, W, W, False, 1.0, 1.0, "silu")
+
+
 def test_raise_for_code_mapping():
     with pytest.raises(TypeError):
         _capi.raise_for_code(_capi.ERR_DTYPE, "x")

@@ -89,3 +89,30 @@ def test_small_decoder_step_matches_the_same_model_on_the_eager_operator():
     m = orc.error_metrics(g_hip.cpu(), model.embed.weight.grad.float().cpu())
     print("embed grad", m, flush=True)
     assert m["mean_rel"] <= 5e-2
+
+
+def test_legacy_single_expert_operator_is_a_per_head_swiglu():
+    """E = 1, R = 1: per head, down(silu(gate(q)) * up(q)) with torch.nn.functional.linear (a library routine, not the
+    oracle), forward and all four gradients; grouped K/U/V heads included."""
+    import torch.nn.functional as F
+    from flashmhf_amd import FlashMLP
+    dev = "cuda:0"
+    torch.manual_seed(11)
+    B, H, Hk, S, dh, I = 2, 4, 2, 150, 128, 192
+    Q = torch.randn(B, H, S, dh).to(torch.bfloat16)
+    K, U, V = ((torch.randn(Hk, I, dh) * dh ** -0.5).to(torch.bfloat16) for _ in range(3))
+    g = torch.randn(B, H, S, dh).to(torch.bfloat16)
+    lv = [t.float().requires_grad_(True) for t in (Q, K, U, V)]
+    outs = []
+    for h in range(H):
+        q, k, u, v = lv[0][:, h], lv[1][h // (H // Hk)], lv[2][h // (H // Hk)], lv[3][h // (H // Hk)]
+        outs.append(F.linear(F.silu(F.linear(q, k)) * F.linear(q, u), v.t()))
+    ref = torch.stack(outs, dim=1)
+    ref.backward(g.float())
+    gl = [t.to(dev).requires_grad_(True) for t in (Q, K, U, V)]
+    out = FlashMLP()(*gl, False, 1.0, 1.0, "silu")
+    out.backward(g.to(dev))
+    torch.cuda.synchronize()
+    _check(out, ref.detach(), "O")
+    for name, a, b in zip(("dQ", "dK", "dU", "dV"), gl, lv):
+        _check(a.grad, b.grad, name)
