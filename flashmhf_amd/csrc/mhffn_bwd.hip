@@ -244,10 +244,8 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     const int e_w = jb_c / p.nbe;
     const long wrow = ((long)hk * nblk + jb_c) * JB + l32;      // this lane's row of K/U/V (column j of the products)
 
-    // K and U blocks stay in (accumulation) registers as MFMA B operands for the whole kernel; the V block of each
-    // wave is parked in LDS (one swizzled tile per wave, behind the ring) and re-read every tile.
-    unsigned char* sVw = smem_raw + DW_NST * DW_STAGE_B + wave * TILE_B;
-    float* sZero = reinterpret_cast<float*>(smem_raw + DW_NST * DW_STAGE_B + 4 * TILE_B);   // 32 zero gate values
+    // The K, U and V blocks stay in registers as MFMA B operands for the whole kernel (K, U in accumulation registers).
+    float* sZero = reinterpret_cast<float*>(smem_raw + DW_NST * DW_STAGE_B);   // 32 zero gate values
     if (tid < 32) sZero[tid] = 0.0f;
     // The first step contracts a tile that does not exist (zero gate values) out of the last stage, which no load has
     // filled yet: clear its Q and dO tiles, or whatever bit patterns the previous kernel left there (possibly NaN or
@@ -257,16 +255,13 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         u32x4* last_stage = reinterpret_cast<u32x4*>(smem_raw + (DW_NST - 1) * DW_STAGE_B);
         for (int i = tid; i < 2 * TILE_B / 16; i += 256) last_stage[i] = z;
     }
-    {
-        const bf16_t* vblk = p.V + (((long)hk * nblk + jb_c) * JB) * DH;
-#pragma unroll
-        for (int ins = 0; ins < 8; ++ins) tile_fill_ins<DH>(vblk, DH, sVw, ins, lane);
-    }
     bf16x8 kB[KS], uB[KS];
+    bf16x8 vR[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         kB[ks] = *reinterpret_cast<const bf16x8*>(p.K + wrow * DH + ks * 16 + 8 * g);
         uB[ks] = *reinterpret_cast<const bf16x8*>(p.U + wrow * DH + ks * 16 + 8 * g);
+        vR[ks] = *reinterpret_cast<const bf16x8*>(p.V + wrow * DH + ks * 16 + 8 * g);
     }
 
     f32x16 dk[CT], du[CT], dv[CT];
@@ -371,13 +366,12 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         const float* pR = live ? reinterpret_cast<const float*>(pG + TILE_B) + wave * 64 : sZero;
 
         bf16x8 pB[2], dmB[2], dnB[2];
-        bf16x8 aq[3], ag[3], vB[3];                  // operand ring: k-step ks+2 is requested while ks is consumed
+        bf16x8 aq[3], ag[3];                         // operand ring: k-step ks+2 is requested while ks is consumed
 #pragma unroll
         for (int k0 = 0; k0 < 2; ++k0) {
             const int off = rowoff + (xg ^ (k0 << 5));
             aq[k0] = *reinterpret_cast<const bf16x8*>(sQ + off);
             ag[k0] = *reinterpret_cast<const bf16x8*>(sG + off);
-            vB[k0] = *reinterpret_cast<const bf16x8*>(sVw + off);
         }
         // gate values of the previous tile for this lane's 16 token rows (4 consecutive rows per 16-byte read)
         f32x4 rv[4];
@@ -440,7 +434,6 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
                 const int off = rowoff + (xg ^ ((ks + 2) << 5));
                 aq[(ks + 2) % 3] = *reinterpret_cast<const bf16x8*>(sQ + off);
                 ag[(ks + 2) % 3] = *reinterpret_cast<const bf16x8*>(sG + off);
-                vB[(ks + 2) % 3] = *reinterpret_cast<const bf16x8*>(sVw + off);
             }
             if constexpr (ks == 0) mfma32_vgpr_first_bacc(m, aq[0], kB[0]);
             else mfma32_vgpr_acc_bacc(m, aq[ks % 3], kB[ks]);
@@ -448,8 +441,8 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
             if constexpr (ks == 0) mfma32_vgpr_first_bacc(n, aq[0], uB[0]);
             else mfma32_vgpr_acc_bacc(n, aq[ks % 3], uB[ks]);
             after_slot1(std::integral_constant<int, 3 * ks + 1>{});
-            if constexpr (ks == 0) mfma32_vgpr_first(da, ag[0], vB[0]);
-            else mfma32_vgpr_acc(da, ag[ks % 3], vB[ks % 3]);
+            if constexpr (ks == 0) mfma32_vgpr_first(da, ag[0], vR[0]);
+            else mfma32_vgpr_acc(da, ag[ks % 3], vR[ks]);
             after_slot1(std::integral_constant<int, 3 * ks + 2>{});
         });
 
@@ -632,7 +625,7 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
     if (phases & 4) {
         DwArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, part,
                  d.B, d.H, G, d.S, d.E, nbe, nslice, d.tokmaj};
-        const int smem = DW_NST * DW_STAGE_B + 4 * TILE_B + 128;
+        const int smem = DW_NST * DW_STAGE_B + 128;
         static bool attr_done = false;   // dynamic LDS above 64 KB must be opted into, per kernel
         if (!attr_done) {
             err = hipFuncSetAttribute((const void*)mhffn_bwd_dkdudv_kernel<DH, false>,
