@@ -56,7 +56,7 @@ def f1(w):
     return 2.0 * w["B"] * w["S"] * w["H"] * w["E"] * w["d_e"] * w["d_h"]
 
 
-def time_events(fn, n, warm=2):
+def time_events(fn, n, warm=10):
     for _ in range(warm):
         fn()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -68,7 +68,7 @@ def time_events(fn, n, warm=2):
     return a.elapsed_time(b) / n
 
 
-def kernel_timings(w, ins, n=10):
+def kernel_timings(w, ins, n=50):
     """Average duration of each kernel, bracketed by events on the launch stream (torch's current stream)."""
     from flashmhf_amd import _capi
     Q, K, U, V, R, dO = ins
@@ -206,8 +206,9 @@ def bench_model(w, args, dev):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50,
+                    help="untimed steps first: the GPU clock needs some tens of milliseconds of load to settle")
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calibrate-copy", action="store_true",
