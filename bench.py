@@ -216,7 +216,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the fused MH-FFN on ONE GPU; --gpus must be 1 "
-              "(heads and tokens shard trivially, see DESIGN.md, but no multi-GPU path is built)", file=sys.stderr)
+              "(heads shard with no exchange and tokens with one all-reduce of dK, dU, dV, but no multi-GPU path is built)", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the fused operator has no CPU path", file=sys.stderr)
