@@ -107,7 +107,7 @@ def kernel_timings(w, ins, n=50):
 CREDIT = {"fwd_main": 3, "bwd_dqdr": 5, "bwd_dkdudv": 3}
 # HBM bytes per launch at workload c2 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy
 # (profiles/c2_hbm_traffic_pmc.md); counters cannot be read from inside this process, so the figures are recorded here.
-TRAFFIC_C2 = {"fwd_main": 122.0e6, "bwd_dqdr": 160.5e6, "bwd_dkdudv": 334.4e6}
+TRAFFIC_C2 = {"fwd_main": 122.2e6, "bwd_dqdr": 160.5e6, "bwd_dkdudv": 334.4e6}
 HARDWARE = {"fwd_main": 3, "bwd_dqdr": 5, "bwd_dkdudv": 6}
 
 
