@@ -609,13 +609,9 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
         const int tokw = NW * 32 * NCT;
         const int smem = DQ_NST * DQ_STAGE_B + d.E * tokw * (int)sizeof(float);
         if (smem > 160 * 1024) return hipErrorInvalidValue;
-        static int attr_smem = 0;   // dynamic LDS above 64 KB must be opted into, per kernel
-        if (smem > attr_smem) {
-            err = hipFuncSetAttribute((const void*)mhffn_bwd_dqdr_kernel<DH, NCT, NW>,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-            if (err != hipSuccess) return err;
-            attr_smem = smem;
-        }
+        static LdsOptIn optin;
+        err = ensure_dynamic_lds(optin, (const void*)mhffn_bwd_dqdr_kernel<DH, NCT, NW>, smem);
+        if (err != hipSuccess) return err;
         dim3 grid((unsigned)d.H, (unsigned)((d.S + tokw - 1) / tokw), (unsigned)d.B);
         hipLaunchKernelGGL((mhffn_bwd_dqdr_kernel<DH, NCT, NW>), grid, dim3(NW * 64), smem, st, a);
         err = hipGetLastError();
@@ -626,17 +622,10 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
         DwArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, part,
                  d.B, d.H, G, d.S, d.E, nbe, nslice, d.tokmaj};
         const int smem = DW_NST * DW_STAGE_B + 128;
-        static bool attr_done = false;   // dynamic LDS above 64 KB must be opted into, per kernel
-        if (!attr_done) {
-            err = hipFuncSetAttribute((const void*)mhffn_bwd_dkdudv_kernel<DH, false>,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-            if (err == hipSuccess)
-                err = hipFuncSetAttribute((const void*)mhffn_bwd_dkdudv_kernel<DH, true>,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-            if (err != hipSuccess) return err;
-            attr_done = true;
-        }
-        if (d.E > 64) return hipErrorInvalidValue;   // staged R tile holds at most 64 experts
+        static LdsOptIn optin_full, optin_tail;
+        err = d.S % 32 == 0 ? ensure_dynamic_lds(optin_full, (const void*)mhffn_bwd_dkdudv_kernel<DH, false>, smem)
+                            : ensure_dynamic_lds(optin_tail, (const void*)mhffn_bwd_dkdudv_kernel<DH, true>, smem);
+        if (err != hipSuccess) return err;
         const int nblk = d.E * nbe;
         dim3 grid((unsigned)d.Hkuv, (unsigned)((nblk + 3) / 4), (unsigned)nslice);
         if (d.S % 32 == 0)

@@ -17,6 +17,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 #include <type_traits>
 
 namespace mhffn {
@@ -236,6 +237,25 @@ template <int N>
 __device__ __forceinline__ void wait_vmcnt()
 {
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+// Dynamic LDS above 64 KB must be opted into per kernel function and per device.  One LdsOptIn per kernel function (static
+// storage, zero-initialised) remembers the largest size already granted on each device, so the attribute call is made
+// once per (kernel, device) whichever host thread launches first; a repeated call is harmless.
+constexpr int LDS_OPTIN_MAX_DEVICES = 64;
+struct LdsOptIn {
+    std::atomic<int> granted[LDS_OPTIN_MAX_DEVICES];
+};
+inline hipError_t ensure_dynamic_lds(LdsOptIn& c, const void* fn, int bytes)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const bool tracked = dev >= 0 && dev < LDS_OPTIN_MAX_DEVICES;
+    if (tracked && bytes <= c.granted[dev].load(std::memory_order_acquire)) return hipSuccess;
+    e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && tracked) c.granted[dev].store(bytes, std::memory_order_release);
+    return e;
 }
 
 // Host-side launch entry points (defined in the per-kernel .hip files).

@@ -288,13 +288,9 @@ hipError_t launch_fwd_f32(const void* Q, const void* K, const void* U, const voi
     a.O = (float*)O;
     a.B = d.B; a.H = d.H; a.G = d.H / d.Hkuv; a.S = d.S; a.DH = d.d_h; a.E = d.E; a.DE = d.d_e; a.tokmaj = d.tokmaj;
     const int smem = (4 * 32 * (d.d_h + 1) + TT * (JC + 1)) * (int)sizeof(float);
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void*)fwd_f32_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           128 * 1024);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    static LdsOptIn optin;
+    const hipError_t e = ensure_dynamic_lds(optin, (const void*)fwd_f32_kernel, 128 * 1024);
+    if (e != hipSuccess) return e;
     dim3 grid((unsigned)d.H, (unsigned)((d.S + TT - 1) / TT), (unsigned)d.B);
     hipLaunchKernelGGL(fwd_f32_kernel, grid, dim3(256), smem, st, a);
     return hipGetLastError();
@@ -309,16 +305,10 @@ hipError_t launch_bwd_f32(const void* Q, const void* K, const void* U, const voi
     a.dO = (const float*)dO; a.dQ = (float*)dQ; a.dR = dR; a.part = (float*)ws;
     a.B = d.B; a.H = d.H; a.G = d.H / d.Hkuv; a.S = d.S; a.DH = d.d_h; a.E = d.E; a.DE = d.d_e; a.tokmaj = d.tokmaj;
     a.nslice = f32_nslice(d);
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void*)dqdr_f32_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           128 * 1024);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute((const void*)dkdudv_f32_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    128 * 1024);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    static LdsOptIn optin_dq, optin_dw;
+    hipError_t e = ensure_dynamic_lds(optin_dq, (const void*)dqdr_f32_kernel, 128 * 1024);
+    if (e == hipSuccess) e = ensure_dynamic_lds(optin_dw, (const void*)dkdudv_f32_kernel, 128 * 1024);
+    if (e != hipSuccess) return e;
     hipError_t err = hipSuccess;
     if (phases & 2) {
         const int smem = (5 * 32 * (d.d_h + 1) + 2 * TT * (JC + 1) + TT * 8) * (int)sizeof(float);

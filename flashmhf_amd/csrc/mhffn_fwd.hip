@@ -234,13 +234,9 @@ static hipError_t launch_fwd_t(const FwdArgs& a, const Dims& d, hipStream_t st)
     const int tokw = 256;
     const int smem = FWD_NST * FWD_STAGE_B + d.E * tokw * (int)sizeof(float);
     if (smem > 160 * 1024) return hipErrorInvalidValue;
-    static int attr_smem = 0;
-    if (smem > attr_smem) {
-        hipError_t e = hipFuncSetAttribute((const void*)mhffn_fwd_kernel<DH>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        attr_smem = smem;
-    }
+    static LdsOptIn optin;
+    const hipError_t e = ensure_dynamic_lds(optin, (const void*)mhffn_fwd_kernel<DH>, smem);
+    if (e != hipSuccess) return e;
     dim3 grid((unsigned)d.H, (unsigned)((d.S + tokw - 1) / tokw), (unsigned)d.B);
     hipLaunchKernelGGL((mhffn_fwd_kernel<DH>), grid, dim3(256), smem, st, a);
     return hipGetLastError();
