@@ -15,6 +15,11 @@ Pinning status (what fixes each function independently of this file's own formul
                                 central finite differences, and the scalar C backward.
   * tk_ground_truth          -- equals mhffn_forward up to rounding (same closed form).
   * mhffn_layer_forward      -- library routines only (F.linear, sigmoid, sum).
+  * mhffn_block_forward      -- library routines around mhffn_forward; with E = 1 (gate identically 1) and no
+                                RMSNorm it equals F.linear -> per-head SwiGLU via F.linear -> F.linear; the per-head
+                                RMSNorm equals F.rms_norm over d_h times the per-head weight; and it agrees with the
+                                independently written flashmhf_amd.mhffn_layer.MHFFNLayer (einsum gate, module
+                                projections) run on the same eager operator.
 The reference holds no golden vectors for this path (it has no tests with stored data), so the
 vectors under tests/golden/ are produced by this oracle after it passed the checks above.
 """

@@ -159,3 +159,29 @@ def test_bf16_eager_is_within_tolerance_of_fp32_oracle():
     got = orc.mhffn_forward(Q, K, U, V, R, compute_dtype=torch.bfloat16, out_dtype=torch.float32)
     m = orc.error_metrics(got, ref)
     assert m["max_abs"] < 2e-2 and m["mean_rel"] < 1e-2
+
+
+def test_block_restatement_reduces_to_library_routines():
+    """mhffn_block_forward: (a) E = 1 makes the gate identically 1, so the block is Linear -> per-head SwiGLU -> Linear,
+    all through F.linear; (b) the per-head RMSNorm inside it is F.rms_norm over d_h times the per-head weight."""
+    import torch.nn.functional as F
+    torch.manual_seed(4)
+    B, S, hid, H, de = 2, 5, 24, 3, 7
+    dh = hid // H
+    x = torch.randn(B, S, hid, dtype=torch.float64)
+    w1, w2 = torch.randn(hid, hid, dtype=torch.float64), torch.randn(hid, hid, dtype=torch.float64)
+    K, U, V = (torch.randn(H, 1, de, dh, dtype=torch.float64) for _ in range(3))
+    router = torch.randn(H, dh, 1, dtype=torch.float64)
+    y = orc.mhffn_block_forward(x, w1, w2, K, U, V, num_heads=H, router=router, compute_dtype=torch.float64)
+    q = F.linear(x, w1).view(B, S, H, dh)
+    heads = [F.linear(F.silu(F.linear(q[:, :, h], K[h, 0])) * F.linear(q[:, :, h], U[h, 0]), V[h, 0].t()) for h in range(H)]
+    ref = F.linear(torch.stack(heads, dim=2).reshape(B, S, hid), w2)
+    assert torch.allclose(y, ref, atol=1e-5, rtol=1e-5)     # the gate is computed in fp32: 1.0 up to fp32 rounding
+
+    g = torch.rand(H, dh, dtype=torch.float64) + 0.5
+    y2 = orc.mhffn_block_forward(x, w1, w2, K, U, V, num_heads=H, router=router, q_norm_weight=g, eps=1e-6,
+                                 compute_dtype=torch.float64)
+    qn = F.rms_norm(q.float(), (dh,), eps=1e-6).double() * g
+    heads = [F.linear(F.silu(F.linear(qn[:, :, h], K[h, 0])) * F.linear(qn[:, :, h], U[h, 0]), V[h, 0].t()) for h in range(H)]
+    ref2 = F.linear(torch.stack(heads, dim=2).reshape(B, S, hid), w2)
+    assert torch.allclose(y2, ref2, atol=1e-4, rtol=1e-4)   # the norm runs in fp32 as the reference's does
