@@ -20,7 +20,7 @@ ERR_NULL_POINTER, ERR_DTYPE, ERR_HEAD_DIM, ERR_EXPERT_DIM, ERR_SHAPE, ERR_WORKSP
 EXPORTS = (
     "mhffn_strerror", "mhffn_is_supported", "mhffn_check_dims", "mhffn_fwd_workspace_bytes",
     "mhffn_bwd_workspace_bytes", "mhffn_fwd", "mhffn_bwd", "mhffn_fwd_phases", "mhffn_bwd_phases",
-    "mhffn_fwd_layout", "mhffn_bwd_layout",
+    "mhffn_fwd_layout", "mhffn_bwd_layout", "mhffn_gate_fwd", "mhffn_gate_bwd",
 )
 TOKENS_BHSD, TOKENS_BSHD = 0, 1     # layout of Q, O, dO, dQ
 FWD_PACK, FWD_MAIN, FWD_ALL = 1, 2, 3
@@ -58,6 +58,8 @@ def lib():
         L.mhffn_fwd_layout.argtypes = [vp] * 6 + [vp, ctypes.c_size_t, dp, ctypes.c_int, ctypes.c_int, vp, ctypes.c_int]
         L.mhffn_bwd_layout.argtypes = ([vp] * 6 + [vp] * 5 + [ctypes.c_int, vp, ctypes.c_size_t, dp, ctypes.c_int,
                                                               ctypes.c_int, vp, ctypes.c_int])
+        L.mhffn_gate_fwd.argtypes = [vp, vp, ctypes.c_float, vp, vp, vp, dp, vp]
+        L.mhffn_gate_bwd.argtypes = [vp, vp, ctypes.c_float, vp, vp, ctypes.c_int, vp, vp, vp, vp, dp, vp]
         _lib = L
     return _lib
 

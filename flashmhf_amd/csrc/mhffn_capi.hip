@@ -153,4 +153,44 @@ int mhffn_bwd(const void* Q, const void* K, const void* U, const void* V, const 
                             dtype, stream, MHFFN_BWD_ALL);
 }
 
+static int check_gate_dims(const mhffn_dims* d)
+{
+    if (!d) return MHFFN_ERR_NULL_POINTER;
+    if (d->B <= 0 || d->H <= 0 || d->S <= 0 || d->E <= 0 || d->d_h <= 0) return MHFFN_ERR_SHAPE;
+    if (d->d_h != 64 && d->d_h != 96 && d->d_h != 128) return MHFFN_ERR_HEAD_DIM;
+    if (d->E > 64 || d->B > 65535 || d->H > 65535 || (long long)d->S > (1ll << 30)) return MHFFN_ERR_SHAPE;
+    if ((long long)d->B * d->H * d->S >= (1ll << 31)) return MHFFN_ERR_SHAPE;
+    return MHFFN_OK;
+}
+
+int mhffn_gate_fwd(const void* X, const float* norm_weight, float eps, const float* router, void* Qn, float* R,
+                   const mhffn_dims* dims, void* stream)
+{
+    const int rc = check_gate_dims(dims);
+    if (rc != MHFFN_OK) return rc;
+    if (!X || !router || !R || (norm_weight && !Qn)) return MHFFN_ERR_NULL_POINTER;
+    if (!aligned16(X) || !aligned16(Qn) || !aligned16(R) || !aligned16(router) || !aligned16(norm_weight))
+        return MHFFN_ERR_ALIGNMENT;
+    return mhffn::launch_gate_fwd(X, norm_weight, eps, router, Qn, R, to_dims(dims), (hipStream_t)stream) == hipSuccess
+               ? MHFFN_OK
+               : MHFFN_ERR_LAUNCH;
+}
+
+int mhffn_gate_bwd(const void* X, const float* norm_weight, float eps, const float* router, const void* dQ,
+                   int dq_token_layout, const float* dR, void* dX, float* d_norm_weight, float* d_router,
+                   const mhffn_dims* dims, void* stream)
+{
+    const int rc = check_gate_dims(dims);
+    if (rc != MHFFN_OK) return rc;
+    if (dq_token_layout != MHFFN_TOKENS_BHSD && dq_token_layout != MHFFN_TOKENS_BSHD) return MHFFN_ERR_SHAPE;
+    if (!X || !router || !dQ || !dR || !dX || !d_router || (norm_weight && !d_norm_weight)) return MHFFN_ERR_NULL_POINTER;
+    const void* ptrs[] = {X, norm_weight, router, dQ, dR, dX, d_norm_weight, d_router};
+    for (const void* p : ptrs)
+        if (!aligned16(p)) return MHFFN_ERR_ALIGNMENT;
+    return mhffn::launch_gate_bwd(X, norm_weight, eps, router, dQ, dq_token_layout, dR, dX, d_norm_weight, d_router,
+                                  to_dims(dims), (hipStream_t)stream) == hipSuccess
+               ? MHFFN_OK
+               : MHFFN_ERR_LAUNCH;
+}
+
 }  // extern "C"

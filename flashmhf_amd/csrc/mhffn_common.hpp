@@ -290,4 +290,10 @@ hipError_t launch_bwd_f32(const void* Q, const void* K, const void* U, const voi
                           void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32, void* ws, const Dims& d,
                           hipStream_t st, int phases);
 
+// Head prologue (mhffn_gate.hip): per-head RMSNorm + expert gate over [B, S, H, d_h] bf16 rows; d_h 64/96/128, E <= 64.
+hipError_t launch_gate_fwd(const void* X, const float* Wn, float eps, const float* Wr, void* Qn, float* R, const Dims& d,
+                           hipStream_t st);
+hipError_t launch_gate_bwd(const void* X, const float* Wn, float eps, const float* Wr, const void* dQ, int dq_tokmaj,
+                           const float* dR, void* dX, float* dWn, float* dWr, const Dims& d, hipStream_t st);
+
 }  // namespace mhffn

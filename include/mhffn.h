@@ -131,6 +131,28 @@ int mhffn_bwd_layout(const void* Q, const void* K, const void* U, const void* V,
                      void* workspace, size_t workspace_bytes,
                      const mhffn_dims* dims, int dtype, int token_layout, void* stream, int phases);
 
+/* Head prologue of the block: what the caller does between its projection and the operator
+ * (models/flashmhf/modeling_mhffnmoe.py:371-372 per-head RMSNorm, class at :97-135; :384-386 expert gate), in one pass
+ * over the projected heads instead of a dozen element-wise passes plus a float32 copy of Q:
+ *
+ *     u = X * rsqrt(mean(X^2 over d_h) + eps)        y = bf16(u * norm_weight[h])          (skipped when norm_weight is NULL)
+ *     z = y . router[h]  (float32)                   s = sigmoid(z)       R = s / max(sum_e s, 1e-20)
+ *
+ *   X, Qn, dX       [B, S, H, d_h] bfloat16: the projection's own memory layout; Qn is the Q to hand to
+ *                   mhffn_fwd_layout(..., MHFFN_TOKENS_BSHD, ...).  With norm_weight NULL, Q is X itself and Qn is not
+ *                   touched (may be NULL).
+ *   norm_weight     [H, d_h] float32 or NULL;  router [H, d_h, E] float32;  R, dR [B, H, S, E] float32.
+ *   dQ              gradient with respect to y, bfloat16, in the layout named by dq_token_layout (MHFFN_TOKENS_*).
+ *   d_norm_weight   [H, d_h] float32 (ignored when norm_weight is NULL), d_router [H, d_h, E] float32: the kernel ADDS
+ *                   its sums over all tokens to what the buffers hold (atomic float adds, so the last bits depend on
+ *                   the order waves finish in); the caller zero-fills them for a plain gradient.
+ * Only dims->B, H, S, d_h, E are read (d_h 64, 96 or 128; E <= 64; B and H at most 65535).  No workspace. */
+int mhffn_gate_fwd(const void* X, const float* norm_weight, float eps, const float* router,
+                   void* Qn, float* R, const mhffn_dims* dims, void* stream);
+int mhffn_gate_bwd(const void* X, const float* norm_weight, float eps, const float* router,
+                   const void* dQ, int dq_token_layout, const float* dR,
+                   void* dX, float* d_norm_weight, float* d_router, const mhffn_dims* dims, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

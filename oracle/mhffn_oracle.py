@@ -20,6 +20,9 @@ Pinning status (what fixes each function independently of this file's own formul
                                 RMSNorm equals F.rms_norm over d_h times the per-head weight; and it agrees with the
                                 independently written flashmhf_amd.mhffn_layer.MHFFNLayer (einsum gate, module
                                 projections) run on the same eager operator.
+  * head_norm_gate           -- F.rms_norm over d_h times the per-head weight, torch.sigmoid and a plain sum (library
+                                routines); rows of R sum to 1; a zero router gives R = 1/E; its gradients are
+                                torch.autograd's and are checked by gradcheck in fp64.
 The reference holds no golden vectors for this path (it has no tests with stored data), so the
 vectors under tests/golden/ are produced by this oracle after it passed the checks above.
 """
@@ -128,6 +131,23 @@ def router_gate(Qh, router):
     models/flashmhf/modeling_mhffnmoe.py:384-386.  Qh [B,H,S,d_h], router [d_h,E] or [H,d_h,E]."""
     R = (Qh.to(torch.float32) @ router.to(torch.float32)).contiguous().sigmoid()
     return R / R.sum(dim=-1, keepdim=True).clamp(min=1e-20)
+
+
+def head_norm_gate(x4, norm_weight, router, eps=1e-6, out_dtype=None):
+    """The block's head prologue, differentiable: per-head RMSNorm in fp32 with the result cast back to the input
+    dtype (models/flashmhf/modeling_mhffnmoe.py:124-133; skipped when norm_weight is None, :371), then the gate from
+    the *rounded* Q in fp32 (:384-386).  x4 [B,S,H,d_h], norm_weight [H,d_h], router [H,d_h,E].
+    Returns Q [B,H,S,d_h] (dtype of x4 unless out_dtype) and R [B,H,S,E] fp32 (or fp64 if x4 is fp64)."""
+    out_dtype = out_dtype or x4.dtype
+    acc = torch.float64 if x4.dtype == torch.float64 else torch.float32
+    q = x4
+    if norm_weight is not None:
+        xf = x4.to(acc)
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+        q = (xf * norm_weight.to(acc).unsqueeze(0).unsqueeze(0)).to(out_dtype)
+    Qh = q.transpose(1, 2)
+    Rs = (Qh.to(acc) @ router.to(acc)).sigmoid()
+    return Qh, Rs / Rs.sum(dim=-1, keepdim=True).clamp(min=1e-20)
 
 
 def mhffn_layer_forward(X, Wq, Wr, K, U, V, Wo, *, num_heads, compute_dtype=torch.float32):

@@ -185,3 +185,27 @@ def test_block_restatement_reduces_to_library_routines():
     heads = [F.linear(F.silu(F.linear(qn[:, :, h], K[h, 0])) * F.linear(qn[:, :, h], U[h, 0]), V[h, 0].t()) for h in range(H)]
     ref2 = F.linear(torch.stack(heads, dim=2).reshape(B, S, hid), w2)
     assert torch.allclose(y2, ref2, atol=1e-4, rtol=1e-4)   # the norm runs in fp32 as the reference's does
+
+
+def test_head_norm_gate_is_pinned_by_library_routines():
+    """Per-head RMSNorm = F.rms_norm over d_h times the per-head weight; gate rows sum to 1; zero router gives 1/E;
+    gradients pass gradcheck in fp64."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(5)
+    B, S, H, dh, E = 2, 5, 3, 8, 4
+    x = torch.randn(B, S, H, dh, generator=g)
+    w = torch.rand(H, dh, generator=g) + 0.5
+    router = torch.randn(H, dh, E, generator=g) * 0.3
+    Q, R = orc.head_norm_gate(x, w, router, eps=1e-5)
+    ref_q = (F.rms_norm(x, (dh,), eps=1e-5) * w).transpose(1, 2)
+    torch.testing.assert_close(Q, ref_q, rtol=1e-6, atol=1e-6)
+    logits = torch.einsum("bhsd,hde->bhse", ref_q, router)
+    ref_R = torch.sigmoid(logits)
+    ref_R = ref_R / ref_R.sum(-1, keepdim=True)
+    torch.testing.assert_close(R, ref_R, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(R.sum(-1), torch.ones(B, H, S), rtol=1e-6, atol=1e-6)
+    Q0, R0 = orc.head_norm_gate(x, None, torch.zeros(H, dh, E))
+    assert torch.equal(Q0, x.transpose(1, 2))
+    torch.testing.assert_close(R0, torch.full((B, H, S, E), 1.0 / E))
+    xd, wd, rd = (t.double().requires_grad_(True) for t in (x[:1, :2], w, router))
+    assert torch.autograd.gradcheck(lambda a, b, c: orc.head_norm_gate(a, b, c, eps=1e-5), (xd, wd, rd), atol=1e-6)
