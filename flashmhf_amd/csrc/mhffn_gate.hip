@@ -201,9 +201,17 @@ __global__ __launch_bounds__(256) void mhffn_gate_fwd_kernel(GateArgs p)
 // ---- backward -------------------------------------------------------------------------------------------------------
 // LDS: router rows (hi, lo) | router columns | norm weight | per wave: y tile (8 KB) + dz tile (8 KB), both in the
 // swizzled 32 x 256-byte tile layout of the main kernels so the transposing reads can be shared.
+// One wave per SIMD (the register partial sums leave no room for a second), so the next tile's rows are requested
+// before the current tile's arithmetic starts; a wave takes enough consecutive tiles that the launch is one wave per
+// SIMD of the chip where the problem allows, which also bounds the number of atomic adds per element.
+// The per-wave region doubles as the staging area of the end-of-kernel reductions over the four waves: one expert
+// tile of d_router partials ((d_h/32) x 16 x 64 floats <= 16 KB) or a 64 x 65 float transpose of the d_norm_weight
+// partials; a [4][128] float array for the latter's cross-wave sums follows the regions.
+constexpr int GATE_WAVE_REGION_B = 2 * TILE_B + 1024;
 constexpr size_t gate_bwd_smem(int DH, int NT)
 {
-    return (size_t)2 * NT * (DH / 16) * 1024 + (size_t)(DH / 32) * 2 * NT * 1024 + DH * 4 + 4 * 2 * TILE_B;
+    return (size_t)2 * NT * (DH / 16) * 1024 + (size_t)(DH / 32) * 2 * NT * 1024 + DH * 4 + 4 * GATE_WAVE_REGION_B +
+           4 * 128 * 4;
 }
 
 template <int CT>
@@ -230,7 +238,8 @@ __global__ __launch_bounds__(256) void mhffn_gate_bwd_kernel(GateArgs p)
     unsigned char* sC = sA + 2 * NT * KS * 1024;                // dy operands
     float* sW = reinterpret_cast<float*>(sC + CT * 2 * NT * 1024);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, g = lane >> 5;
-    unsigned char* ytile = reinterpret_cast<unsigned char*>(sW + DH) + wave * 2 * TILE_B;
+    unsigned char* regions = reinterpret_cast<unsigned char*>(sW + DH);
+    unsigned char* ytile = regions + wave * GATE_WAVE_REGION_B;
     unsigned char* ztile = ytile + TILE_B;
     const int h = blockIdx.y, b = blockIdx.z;
 
@@ -260,31 +269,48 @@ __global__ __launch_bounds__(256) void mhffn_gate_bwd_kernel(GateArgs p)
     const int ntiles = (p.S + 31) / 32;
     const int tile0 = (blockIdx.x * 4 + wave) * p.tpw;
     const int tile1 = min(tile0 + p.tpw, ntiles);
-    for (int tile = tile0; tile < tile1; ++tile) {
+    // rows of the tile after the current one, requested one iteration ahead
+    u32x4 nx[KS], ndq[KS];
+    float ngr[NT][16];
+    auto request = [&](int tile) {
         const int t = tile * 32 + l32;
         const bool valid = t < p.S;
         const int tc = valid ? t : p.S - 1;
-        const long row = (((long)b * p.S + tc) * p.H + h) * DH;
+        const bf16_t* xrow = p.X + (((long)b * p.S + tc) * p.H + h) * DH;
+        const bf16_t* dqrow = p.dQ + (dqrows.base + (long)tc * dqrows.stride) * DH;
+        const float* drow = p.dR + (((long)b * p.H + h) * p.S + tc) * p.E;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            nx[ks] = *reinterpret_cast<const u32x4*>(xrow + (2 * ks + g) * 8);
+            ndq[ks] = *reinterpret_cast<const u32x4*>(dqrow + (2 * ks + g) * 8);
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int e = nt * 32 + 16 * (i >> 3) + 8 * g + (i & 7);
+                ngr[nt][i] = (valid && e < p.E) ? drow[e] : 0.0f;
+            }
+    };
+    if (tile0 < tile1) request(tile0);
+    for (int tile = tile0; tile < tile1; ++tile) {
+        const int t = tile * 32 + l32;
+        const bool valid = t < p.S;
+        const long row = (((long)b * p.S + (valid ? t : p.S - 1)) * p.H + h) * DH;
         GateTile<DH, NT, NORM> T;
         T.eps_ = p.eps;
-        T.load(p.X + row, g);
         u32x4 dqr[KS];
-        {
-            const bf16_t* dqrow = p.dQ + (dqrows.base + (long)tc * dqrows.stride) * DH;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) dqr[ks] = *reinterpret_cast<const u32x4*>(dqrow + (2 * ks + g) * 8);
-        }
         float gr[NT][16];
-        {
-            const float* drow = p.dR + (((long)b * p.H + h) * p.S + tc) * p.E;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int e = nt * 32 + 16 * (i >> 3) + 8 * g + (i & 7);
-                    gr[nt][i] = (valid && e < p.E) ? drow[e] : 0.0f;
-                }
+        for (int ks = 0; ks < KS; ++ks) {
+            T.xr[ks] = nx[ks];
+            dqr[ks] = ndq[ks];
         }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) gr[nt][i] = ngr[nt][i];
+        if (tile + 1 < tile1) request(tile + 1);
         T.normalise(sW, g);
         if (!valid) {   // rows past the end contribute nothing to the sums over tokens
 #pragma unroll
@@ -384,46 +410,70 @@ __global__ __launch_bounds__(256) void mhffn_gate_bwd_kernel(GateArgs p)
         }
     }
 
-    if (tile0 >= tile1) return;
+    // ---- sums over tokens: the four waves' partials meet in LDS, then one atomic add per workgroup and element ------
+    __syncthreads();   // every wave is past its last tile: the per-wave regions are free
+    float* mine = reinterpret_cast<float*>(regions + wave * GATE_WAVE_REGION_B);
     float* dWr = p.dWr + (long)h * DH * p.E;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        const int e = nt * 32 + l32;
-        if (e < p.E)
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct)
+        for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    unsafeAtomicAdd(dWr + (long)(ct * 32 + 8 * (i >> 2) + 4 * g + (i & 3)) * p.E + e, wacc[ct][nt][i]);
+            for (int i = 0; i < 16; ++i) mine[(ct * 16 + i) * 64 + lane] = wacc[ct][nt][i];
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < CT * 16 * 64; idx += 256) {
+            float v = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) v += reinterpret_cast<const float*>(regions + w * GATE_WAVE_REGION_B)[idx];
+            const int ln = idx & 63, i = (idx >> 6) & 15, ct = idx >> 10;
+            const int e = nt * 32 + (ln & 31), col = ct * 32 + 8 * (i >> 2) + 4 * (ln >> 5) + (i & 3);
+            if (e < p.E) unsafeAtomicAdd(dWr + (long)col * p.E + e, v);
+        }
+        __syncthreads();
     }
     if constexpr (NORM) {
+        // transpose inside the wave: value v = 8 ks + j of every lane goes to row v (row stride 65 floats keeps both the
+        // writes and the row-wise reads conflict-free), then lane v adds up each lane half of its row
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                float v = dwacc[ks][j];
-#pragma unroll
-                for (int off = 16; off >= 1; off >>= 1) v += __shfl_xor(v, off);
-                if (l32 == 0) unsafeAtomicAdd(p.dWn + h * DH + (2 * ks + g) * 8 + j, v);
+            for (int j = 0; j < 8; ++j) mine[(ks * 8 + j) * 65 + lane] = dwacc[ks][j];
+        float* cross = reinterpret_cast<float*>(regions + 4 * GATE_WAVE_REGION_B);   // [4 waves][128 columns]
+        if (lane < KS * 8) {
+            float s0 = 0.0f, s1 = 0.0f;
+            for (int i = 0; i < 32; ++i) {
+                s0 += mine[lane * 65 + i];
+                s1 += mine[lane * 65 + 32 + i];
             }
+            const int ks = lane >> 3, j = lane & 7;
+            cross[wave * 128 + (2 * ks) * 8 + j] = s0;
+            cross[wave * 128 + (2 * ks + 1) * 8 + j] = s1;
+        }
+        __syncthreads();
+        if (threadIdx.x < DH)
+            unsafeAtomicAdd(p.dWn + h * DH + threadIdx.x, cross[threadIdx.x] + cross[128 + threadIdx.x] +
+                                                              cross[256 + threadIdx.x] + cross[384 + threadIdx.x]);
     }
 }
 
 // ---- launch ---------------------------------------------------------------------------------------------------------
 namespace {
 
-int tiles_per_wave(const GateArgs& a)
+int tiles_per_wave(const GateArgs& a, bool backward)
 {
     const long total = (long)a.B * a.H * ((a.S + 31) / 32);
-    long tpw = total / 8192;   // aim for at least 8 waves per SIMD over the launch before a wave takes several tiles
-    return (int)(tpw < 1 ? 1 : tpw > 16 ? 16 : tpw);
+    // forward: several waves per SIMD hide the latency, so a wave only takes several tiles once there are at least 8 waves
+    // per SIMD; backward: one wave per SIMD with its own prefetch, as few waves (= atomic adds) as fill the chip once
+    const long tpw = backward ? total / 1024 : total / 8192;
+    const long cap = backward ? 64 : 16;
+    return (int)(tpw < 1 ? 1 : tpw > cap ? cap : tpw);
 }
 
 template <int DH, int NT, bool NORM>
 hipError_t launch_gate(GateArgs a, bool backward, hipStream_t st)
 {
     static LdsOptIn optin_fwd, optin_bwd;
-    a.tpw = tiles_per_wave(a);
+    a.tpw = tiles_per_wave(a, backward);
     const int ntiles = (a.S + 31) / 32;
     const dim3 grid((ntiles + 4 * a.tpw - 1) / (4 * a.tpw), a.H, a.B);
     if (backward) {

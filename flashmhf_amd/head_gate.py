@@ -45,14 +45,14 @@ class HeadNormGateFunction(torch.autograd.Function):
         rc = _capi.lib().mhffn_gate_fwd(x4.data_ptr(), _ptr(wn), float(eps), wr.data_ptr(), _ptr(qn), R.data_ptr(),
                                         dims, torch.cuda.current_stream(x4.device).cuda_stream)
         _capi.raise_for_code(rc, "mhffn_gate_fwd")
-        ctx.save_for_backward(x4, norm_weight, router)
+        ctx.save_for_backward(x4, norm_weight, router, wn, wr)
         ctx.eps = float(eps)
         Q = (qn if qn is not None else x4).transpose(1, 2)
         return Q, R
 
     @staticmethod
     def backward(ctx, dQ, dR):
-        x4, norm_weight, router = ctx.saved_tensors
+        x4, norm_weight, router, wn, wr = ctx.saved_tensors
         dims = _check(x4, norm_weight, router)
         if dQ is None:
             dQ = torch.zeros_like(x4).transpose(1, 2)
@@ -63,8 +63,6 @@ class HeadNormGateFunction(torch.autograd.Function):
         else:
             layout, dQ = _capi.TOKENS_BHSD, dQ.contiguous()
         dR = dR.float().contiguous()
-        wn = None if norm_weight is None else norm_weight.detach().float().contiguous()
-        wr = router.detach().float().contiguous()
         dx = torch.empty_like(x4)
         dwn = None if wn is None else torch.zeros_like(wn)
         dwr = torch.zeros_like(wr)

@@ -14,6 +14,10 @@ but laid out for the HIP kernels instead of for the Triton ones:
 * Q stays in the ``[B, S, H, d_h]`` memory the projection wrote and O comes back in it, so neither of the two
   transposes-with-copy around the operator (:374, :408) happens.
 
+* with bfloat16 activations and ``router_input="q"`` the per-head RMSNorm and the gate run as one HIP pass over the
+  projection's output (``head_gate.head_norm_gate``) instead of a dozen element-wise kernels and a float32 copy of Q;
+  ``fused_prologue=False`` keeps the plain torch operations (the only path for float32 activations).
+
 ``router_input="q"`` takes the gate logits from the per-head Q through ``router [H, d_h, E]`` as the reference model
 does; ``router_input="x"`` takes them from the block input through ``w_router [hid, H*E]``, which is how the layer
 benchmark configurations state the gate.
@@ -30,6 +34,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from .flash_mlp_moe import FlashMLPMoE
+from .head_gate import head_norm_gate
 
 
 class RMSNorm(nn.Module):
@@ -57,7 +62,7 @@ def router_gate(logits):
 
 class MHFFNLayer(nn.Module):
     def __init__(self, hidden_size, num_heads, num_experts, expert_dim, num_kuv_heads=None, *, apply_rmsnorm=False,
-                 rms_norm_eps=1e-6, bias=False, router_input="q", op=None):
+                 rms_norm_eps=1e-6, bias=False, router_input="q", op=None, fused_prologue=True):
         super().__init__()
         if hidden_size % num_heads:
             raise ValueError("hidden_size must be a multiple of num_heads")
@@ -68,6 +73,8 @@ class MHFFNLayer(nn.Module):
         self.head_dim = hidden_size // num_heads
         self.num_experts, self.expert_dim = num_experts, expert_dim
         self.router_input = router_input
+        self.fused_prologue = fused_prologue
+        self.rms_norm_eps = rms_norm_eps
         self.w_self = nn.Linear(hidden_size, hidden_size, bias=bias)
         self.w_self_2 = nn.Linear(hidden_size, hidden_size, bias=bias)
         wshape = (self.num_kuv_heads, num_experts, expert_dim, self.head_dim)
@@ -95,6 +102,10 @@ class MHFFNLayer(nn.Module):
         B, S, _ = x.shape
         H, dh, E = self.num_heads, self.head_dim, self.num_experts
         q = self.w_self(x).view(B, S, H, dh)
+        if (self.fused_prologue and self.router_input == "q" and q.dtype == torch.bfloat16 and q.is_cuda
+                and E <= 64 and dh in (64, 96, 128)):
+            return head_norm_gate(q, None if self.q_norm is None else self.q_norm.weight, self.router,
+                                  self.rms_norm_eps)
         if self.q_norm is not None:
             q = self.q_norm(q)
         Q = q.transpose(1, 2)                                       # a view: the kernels read token-major rows
