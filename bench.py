@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused multi-head FFN hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3|c4] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3|c4|c2_prologue|c3_prologue] [--no-cpu]
 
 One "step" = one forward + one backward of the fused operator (through the C ABI, on torch's current stream) over
 one synthetic batch already resident in HBM.  Prints ONE JSON line.  Credited FLOPs: F1 = 2*T*H*E*d_e*d_h per
@@ -11,6 +11,11 @@ that (the two-kernel backward runs 11*F1 on the hardware, 14*F1 with the forward
 Workload c4 is different in kind: one forward + backward of a whole random-init decoder (20 blocks of causal attention +
 the MH-FFN block of workload c3's shape, vocabulary 50,304) on batch 2 x 4096 random token ids; it reports tokens/s and
 peak memory only.
+
+Workloads c2_prologue / c3_prologue time the block's head prologue (per-head RMSNorm + expert gate, forward and backward,
+mhffn_gate_fwd / mhffn_gate_bwd) on the [B,S,H,d_h] heads of workloads c2 / c3.  These kernels are bound by HBM traffic:
+the value is algorithmic bytes per second, forward 2|Q| + |R| (read x, write Q and R), backward 3|Q| + |R| (read x, dQ
+and dR, write dx), |Q| = 2 T H d_h, |R| = 4 T H E; the router and norm weights and their gradients are a few KB per head.
 """
 import argparse
 import json
@@ -24,6 +29,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
 
 WORKLOADS = {
     # name: (B, S, hidden, H, d_h, E, d_e, passes)
@@ -34,6 +40,12 @@ WORKLOADS = {
     "c4": dict(B=2, S=4096, H=16, d_h=128, E=22, d_e=352, layers=20, vocab=50304, attn_heads=16, passes="model",
                label="1.3B decoder (20 blocks: causal MHA + MH-FFN H16 d_h128 E22 d_e352, RMSNorm, vocab 50304), "
                      "one bf16 forward+backward, B2xS4096 random token ids"),
+    "c2_prologue": dict(B=8, S=2048, H=8, d_h=128, E=11, passes="prologue",
+                        label="head prologue (per-head RMSNorm + expert gate) fwd+bwd on the 370M layer's heads, bf16, "
+                              "B8xS2048 tokens, H8 d_h128 E11"),
+    "c3_prologue": dict(B=4, S=8192, H=16, d_h=128, E=22, passes="prologue",
+                        label="head prologue (per-head RMSNorm + expert gate) fwd+bwd on the 1.3B layer's heads, bf16, "
+                              "B4xS8192 tokens, H16 d_h128 E22"),
 }
 
 
@@ -203,6 +215,83 @@ def bench_model(w, args, dev):
     print(json.dumps(out))
 
 
+def bench_prologue(w, args, dev):
+    """Head prologue kernels through the C ABI on preallocated buffers: one step = forward + backward."""
+    from flashmhf_amd import _capi
+    B, S, H, dh, E = (w[k] for k in ("B", "S", "H", "d_h", "E"))
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(B, S, H, dh, generator=g).bfloat16().to(dev)
+    wn = (torch.rand(H, dh, generator=g) + 0.5).to(dev)
+    wr = (torch.randn(H, dh, E, generator=g) * 0.02 * (H * dh) ** 0.5 / dh ** 0.5).to(dev)
+    dQ = torch.randn(B, S, H, dh, generator=g).bfloat16().to(dev)
+    dR = torch.randn(B, H, S, E, generator=g).to(dev)
+    Qn, dX = torch.empty_like(x), torch.empty_like(x)
+    R = torch.empty(B, H, S, E, device=dev)
+    dwn, dwr = torch.zeros_like(wn), torch.zeros_like(wr)
+    L = _capi.lib()
+    dims = _capi.Dims(B, H, H, S, dh, E, 32)
+    st = torch.cuda.current_stream().cuda_stream
+
+    def fwd():
+        rc = L.mhffn_gate_fwd(x.data_ptr(), wn.data_ptr(), 1e-6, wr.data_ptr(), Qn.data_ptr(), R.data_ptr(), dims, st)
+        assert rc == 0, rc
+
+    def bwd():
+        rc = L.mhffn_gate_bwd(x.data_ptr(), wn.data_ptr(), 1e-6, wr.data_ptr(), dQ.data_ptr(), _capi.TOKENS_BSHD,
+                              dR.data_ptr(), dX.data_ptr(), dwn.data_ptr(), dwr.data_ptr(), dims, st)
+        assert rc == 0, rc
+
+    def step():
+        fwd()
+        bwd()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    q_bytes, r_bytes = 2.0 * B * S * H * dh, 4.0 * B * S * H * E
+    alg = {"gate_fwd": 2 * q_bytes + r_bytes, "gate_bwd": 3 * q_bytes + r_bytes}
+    kt = {"gate_fwd": time_events(fwd, 50), "gate_bwd": time_events(bwd, 50)}
+    dom = max(kt, key=kt.get)
+    ach = alg[dom] / (kt[dom] * 1e-3) / 1e9
+    out = {
+        "metric": "MH-FFN head prologue fwd+bwd GB/s (algorithmic bytes), 1 GPU", "value": sum(alg.values()) / (ms * 1e-3) / 1e9,
+        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {w['label']}", "algorithmic_bytes_per_step": sum(alg.values())},
+        "tokens_per_s": B * S / (ms * 1e-3),
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": ach / PEAK_HBM_GBS, "traffic": None},
+        "kernels": {k: {"ms": v, "algorithmic_gbs": alg[k] / (v * 1e-3) / 1e9} for k, v in kt.items()},
+    }
+    if not args.no_cpu:
+        from oracle import mhffn_oracle as orc
+        xs = x[:1, :1024].float().cpu().requires_grad_(True)
+        wns, wrs = wn.cpu().requires_grad_(True), wr.cpu().requires_grad_(True)
+        dQs, dRs = dQ[:1, :1024].float().cpu().transpose(1, 2), dR[:1, :, :1024].cpu()
+
+        def run():
+            q, r = orc.head_norm_gate(xs, wns, wrs)
+            torch.autograd.grad([q, r], [xs, wns, wrs], [dQs, dRs])
+
+        run()
+        times = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            run()
+            times.append(time.perf_counter() - t0)
+        med = sorted(times)[2]
+        frac = 1024.0 / (B * S)
+        out["cpu_baseline"] = {"value": sum(alg.values()) * frac / med / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "sample": f"oracle head_norm_gate + autograd, fp32, B1xS1024 tokens of the "
+                                                         f"same heads, median of 5 runs, {med * 1e3:.1f} ms"}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -234,6 +323,8 @@ def main():
     w = WORKLOADS[args.workload]
     if w["passes"] == "model":
         return bench_model(w, args, dev)
+    if w["passes"] == "prologue":
+        return bench_prologue(w, args, dev)
     ins = make_inputs(w, dev)
     Q, K, U, V, R, dO = ins
     bwd = "bwd" in w["passes"]

@@ -150,7 +150,9 @@ struct GateTile {
     float eps_;
 };
 
-constexpr size_t gate_fwd_smem(int DH, int NT) { return (size_t)2 * NT * (DH / 16) * 1024 + DH * 4; }
+// router operands | norm weight | per wave: a [32 tokens][E] float tile of R, so that the 32 x E block (contiguous in
+// memory) leaves the wave as whole cache lines instead of one scattered dword per lane and expert
+constexpr size_t gate_fwd_smem(int DH, int NT) { return (size_t)2 * NT * (DH / 16) * 1024 + DH * 4 + 4 * TILE_B; }
 
 template <int DH, int NT, bool NORM>
 __global__ __launch_bounds__(256) void mhffn_gate_fwd_kernel(GateArgs p)
@@ -159,6 +161,7 @@ __global__ __launch_bounds__(256) void mhffn_gate_fwd_kernel(GateArgs p)
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float* sW = reinterpret_cast<float*>(smem + 2 * NT * KS * 1024);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, g = lane >> 5;
+    float* rtile = sW + DH + wave * (TILE_B / 4);
     const int h = blockIdx.y, b = blockIdx.z;
 
     stage_router_rows<DH, NT>(p.Wr + (long)h * DH * p.E, p.E, smem);
@@ -185,16 +188,16 @@ __global__ __launch_bounds__(256) void mhffn_gate_fwd_kernel(GateArgs p)
             }
         }
         T.gate(smem, lane, g, p.E);
-        if (valid) {
-            float* rrow = p.R + (((long)b * p.H + h) * p.S + t) * p.E;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
+        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int e = nt * 32 + 16 * (i >> 3) + 8 * g + (i & 7);
-                    if (e < p.E) rrow[e] = T.s[nt][i] * T.inv;
-                }
-        }
+            for (int i = 0; i < 16; ++i) {
+                const int e = nt * 32 + 16 * (i >> 3) + 8 * g + (i & 7);
+                if (e < p.E) rtile[l32 * p.E + e] = T.s[nt][i] * T.inv;
+            }
+        float* rblock = p.R + (((long)b * p.H + h) * p.S + tile * 32) * p.E;
+        const int lim = min(32, p.S - tile * 32) * p.E;
+        for (int idx = lane; idx < lim; idx += 64) rblock[idx] = rtile[idx];
     }
 }
 
@@ -271,26 +274,23 @@ __global__ __launch_bounds__(256) void mhffn_gate_bwd_kernel(GateArgs p)
     const int tile1 = min(tile0 + p.tpw, ntiles);
     // rows of the tile after the current one, requested one iteration ahead
     u32x4 nx[KS], ndq[KS];
-    float ngr[NT][16];
+    float ngr[NT * 16];
     auto request = [&](int tile) {
         const int t = tile * 32 + l32;
         const bool valid = t < p.S;
         const int tc = valid ? t : p.S - 1;
         const bf16_t* xrow = p.X + (((long)b * p.S + tc) * p.H + h) * DH;
         const bf16_t* dqrow = p.dQ + (dqrows.base + (long)tc * dqrows.stride) * DH;
-        const float* drow = p.dR + (((long)b * p.H + h) * p.S + tc) * p.E;
+        const float* dblock = p.dR + (((long)b * p.H + h) * p.S + tile * 32) * p.E;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             nx[ks] = *reinterpret_cast<const u32x4*>(xrow + (2 * ks + g) * 8);
             ndq[ks] = *reinterpret_cast<const u32x4*>(dqrow + (2 * ks + g) * 8);
         }
+        // the tile's [32][E] block of dR is contiguous: dword k*64 + lane of it, zero past the last token
+        const int lim = min(32, p.S - tile * 32) * p.E;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int e = nt * 32 + 16 * (i >> 3) + 8 * g + (i & 7);
-                ngr[nt][i] = (valid && e < p.E) ? drow[e] : 0.0f;
-            }
+        for (int k = 0; k < NT * 16; ++k) ngr[k] = k * 64 + lane < lim ? dblock[k * 64 + lane] : 0.0f;
     };
     if (tile0 < tile1) request(tile0);
     for (int tile = tile0; tile < tile1; ++tile) {
@@ -306,10 +306,19 @@ __global__ __launch_bounds__(256) void mhffn_gate_bwd_kernel(GateArgs p)
             T.xr[ks] = nx[ks];
             dqr[ks] = ndq[ks];
         }
+        // dR goes lane-major -> token-major through the (currently idle) dz tile
+        {
+            float* rt = reinterpret_cast<float*>(ztile);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+            for (int k = 0; k < NT * 16; ++k) rt[k * 64 + lane] = ngr[k];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) gr[nt][i] = ngr[nt][i];
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int e = nt * 32 + 16 * (i >> 3) + 8 * g + (i & 7);
+                    gr[nt][i] = e < p.E ? rt[l32 * p.E + e] : 0.0f;
+                }
+        }
         if (tile + 1 < tile1) request(tile + 1);
         T.normalise(sW, g);
         if (!valid) {   // rows past the end contribute nothing to the sums over tokens
