@@ -19,13 +19,13 @@ def _check(x4, norm_weight, router):
         raise RuntimeError("expected x [B,S,H,d_h] and router [H,d_h,E]")
     if x4.dtype != torch.bfloat16:
         raise TypeError(f"head_norm_gate expects bfloat16 heads, got {x4.dtype}")
-    if not x4.is_cuda:
-        raise RuntimeError("flashmhf_amd runs on the GPU only; there is no CPU path")
     B, S, H, dh = x4.shape
     if router.shape[:2] != (H, dh):
         raise RuntimeError(f"router must be [H,d_h,E] = [{H},{dh},E], got {tuple(router.shape)}")
     if norm_weight is not None and norm_weight.shape != (H, dh):
         raise RuntimeError(f"norm_weight must be [H,d_h] = [{H},{dh}], got {tuple(norm_weight.shape)}")
+    if not x4.is_cuda:
+        raise RuntimeError("flashmhf_amd runs on the GPU only; there is no CPU path")
     return _capi.Dims(B, H, H, S, dh, router.shape[2], 32)
 
 

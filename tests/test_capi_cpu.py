@@ -87,6 +87,36 @@ def test_entry_points_validate_before_touching_the_gpu(L):
     assert L.mhffn_check_dims(huge, 0) == _capi.ERR_SHAPE
 
 
+def test_gate_entry_points_validate_before_touching_the_gpu(L):
+    d = _capi.Dims(1, 2, 2, 64, 128, 2, 32)
+    null, ok, odd = ctypes.c_void_p(0), ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1004)
+    assert L.mhffn_gate_fwd(null, null, 1e-6, null, null, null, d, null) == _capi.ERR_NULL_POINTER
+    assert L.mhffn_gate_fwd(ok, ok, 1e-6, ok, null, ok, d, null) == _capi.ERR_NULL_POINTER     # norm weight without Qn
+    assert L.mhffn_gate_fwd(ok, ok, 1e-6, ok, odd, ok, d, null) == _capi.ERR_ALIGNMENT
+    assert L.mhffn_gate_fwd(ok, ok, 1e-6, ok, ok, ok, _capi.Dims(1, 2, 2, 64, 100, 2, 32), null) == _capi.ERR_HEAD_DIM
+    assert L.mhffn_gate_fwd(ok, ok, 1e-6, ok, ok, ok, _capi.Dims(1, 2, 2, 64, 128, 65, 32), null) == _capi.ERR_SHAPE
+    assert L.mhffn_gate_fwd(ok, ok, 1e-6, ok, ok, ok, _capi.Dims(1, 70000, 2, 64, 128, 2, 32), null) == _capi.ERR_SHAPE
+    assert L.mhffn_gate_bwd(ok, ok, 1e-6, ok, ok, 0, ok, ok, null, ok, d, null) == _capi.ERR_NULL_POINTER   # norm without its grad
+    assert L.mhffn_gate_bwd(ok, ok, 1e-6, ok, ok, 5, ok, ok, ok, ok, d, null) == _capi.ERR_SHAPE
+    assert L.mhffn_gate_bwd(ok, ok, 1e-6, ok, ok, 1, ok, odd, ok, ok, d, null) == _capi.ERR_ALIGNMENT
+    assert L.mhffn_gate_bwd(ok, ok, 1e-6, ok, ok, 1, ok, ok, ok, ok, None, null) == _capi.ERR_NULL_POINTER
+
+
+def test_head_gate_python_boundary_checks():
+    import torch
+    from flashmhf_amd.head_gate import head_norm_gate
+    x = torch.zeros(1, 4, 2, 128, dtype=torch.bfloat16)
+    router = torch.zeros(2, 128, 3)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        head_norm_gate(x, None, router)
+    with pytest.raises(TypeError):
+        head_norm_gate(x.float(), None, router)
+    with pytest.raises(RuntimeError, match="router must be"):
+        head_norm_gate(x, None, torch.zeros(3, 128, 3))
+    with pytest.raises(RuntimeError, match="norm_weight must be"):
+        head_norm_gate(x, torch.zeros(2, 64), router)
+
+
 def test_python_boundary_raises_reference_exception_types():
     from flashmhf_amd import FlashFFNMoE, FlashMLPMoE
     Q = torch.zeros(1, 2, 8, 128, dtype=torch.bfloat16)

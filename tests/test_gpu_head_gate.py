@@ -95,3 +95,54 @@ def test_gate_backward_matches_autograd_of_oracle(B, S, H, dh, E, norm, token_ma
         assert m["max_abs"] <= 2e-2 * scale, (name, m)
         if ref.abs().max().item() > 1e-4:      # E = 1 makes the gate identically 1: its gradients are rounding noise
             assert m["mean_rel"] <= 1e-2, (name, m)
+
+
+def test_gate_backward_accumulates_into_weight_gradients():
+    """d_router and d_norm_weight are added to what the buffers hold: a second call doubles them; dx is overwritten."""
+    from flashmhf_amd import _capi
+    B, S, H, dh, E = 2, 100, 3, 96, 7
+    x, w, router = _inputs(B, S, H, dh, E, True, seed=3)
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(4)
+    xd, wd, rd = x.to(dev), w.float().to(dev), router.float().to(dev)
+    dQ = torch.randn(B, S, H, dh, generator=g).bfloat16().to(dev)
+    dR = torch.randn(B, H, S, E, generator=g).to(dev)
+    dx = torch.empty_like(xd)
+    dwn, dwr = torch.zeros_like(wd), torch.zeros_like(rd)
+    L, dims, st = _capi.lib(), _capi.Dims(B, H, H, S, dh, E, 32), torch.cuda.current_stream().cuda_stream
+
+    def call():
+        rc = L.mhffn_gate_bwd(xd.data_ptr(), wd.data_ptr(), 1e-6, rd.data_ptr(), dQ.data_ptr(), _capi.TOKENS_BSHD,
+                              dR.data_ptr(), dx.data_ptr(), dwn.data_ptr(), dwr.data_ptr(), dims, st)
+        assert rc == 0, rc
+        torch.cuda.synchronize()
+
+    call()
+    dx1, dwn1, dwr1 = dx.clone(), dwn.clone(), dwr.clone()
+    call()
+    assert torch.equal(dx, dx1)
+    torch.testing.assert_close(dwn, 2 * dwn1, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(dwr, 2 * dwr1, rtol=1e-5, atol=1e-6)
+
+
+def test_layer_with_and_without_the_fused_prologue_agree():
+    from flashmhf_amd import MHFFNLayer
+    torch.manual_seed(0)
+    dev = "cuda:0"
+    layer = MHFFNLayer(256, 2, 4, 64, apply_rmsnorm=True).to(dev).bfloat16()
+    with torch.no_grad():
+        layer.q_norm.weight.uniform_(0.5, 1.5)
+        layer.router.normal_(0, 0.2)
+    x = torch.randn(2, 70, 256, device=dev).bfloat16()
+    outs = []
+    for fused in (True, False):
+        layer.fused_prologue = fused
+        layer.zero_grad(set_to_none=True)
+        xi = x.clone().requires_grad_(True)
+        y = layer(xi)
+        y.float().square().mean().backward()
+        outs.append((y.detach().float(), xi.grad.float(), layer.router.grad.float(), layer.q_norm.weight.grad.float(),
+                     layer.w_self.weight.grad.float()))
+    for name, a, b in zip(("y", "dx", "d_router", "d_q_norm", "d_w_self"), *outs):
+        scale = max(b.abs().max().item(), 1e-6)
+        assert (a - b).abs().max().item() <= 3e-2 * scale, (name, (a - b).abs().max().item(), scale)
