@@ -351,6 +351,27 @@ def main():
     tflops = flops / (ms * 1e-3) / 1e12
     tokens = w["B"] * w["S"]
 
+    # per-step spread (one event pair per step) and the same step through the autograd operator
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(min(args.steps, 100))]
+    for a, b in evs:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    per_step = sorted(a.elapsed_time(b) for a, b in evs)
+    timing = {"median_ms": per_step[len(per_step) // 2], "min_ms": per_step[0]}
+    if bwd:
+        from flashmhf_amd import FlashMLPMoE
+        op = FlashMLPMoE()
+        leaves = [t.detach().clone().requires_grad_(True) for t in (Q, K, U, V, R)]
+
+        def autograd_step():
+            for t in leaves:
+                t.grad = None
+            op(*leaves).backward(dO)
+
+        timing["autograd_op_ms"] = time_events(autograd_step, min(args.steps, 100))
+
     kt = kernel_timings(w, ins)
     dom = max(CREDIT, key=lambda k: kt.get(k, 0.0))
     ach = CREDIT[dom] * f1(w) / (kt[dom] * 1e-3) / 1e12
@@ -375,6 +396,7 @@ def main():
                            "forbidden_intermediate_bytes_one_tensor": tokens * w["H"] * w["E"] * w["d_e"] * 2},
         "roofline": roofline,
         "kernels": kernels,
+        "timing": timing,
     }
     if args.workload == "c3":
         out["swiglu_2048_5504_peak_hbm_bytes_beyond_inputs"] = swiglu_peak_bytes(tokens, 2048, 5504, dev)
