@@ -114,6 +114,24 @@ def kernel_timings(w, ins, n=50):
     return out
 
 
+def measured_mfma_peak_tflops(dev):
+    """Rate of a register-resident v_mfma_f32_32x32x16_bf16 loop on every SIMD (mhffn_probe_mfma_peak), ~5 ms per launch."""
+    import ctypes
+    from flashmhf_amd import _capi
+    L = _capi.lib()
+    sink = torch.zeros(4, device=dev)
+    flops = ctypes.c_double(0.0)
+    blocks = torch.cuda.get_device_properties(dev).multi_processor_count
+    st = torch.cuda.current_stream().cuda_stream
+
+    def run():
+        rc = L.mhffn_probe_mfma_peak(sink.data_ptr(), blocks, 10000, st, ctypes.byref(flops))
+        assert rc == 0, rc
+
+    ms = time_events(run, 5, warm=3)
+    return flops.value / (ms * 1e-3) / 1e12
+
+
 # Credited GEMMs per kernel (in units of F1): the forward's three; the dQ/dR kernel's recomputed M, N, dA and the two
 # dQ products; the dK/dU/dV kernel's three output products (its own recomputation of M, N, dA is not credited).
 CREDIT = {"fwd_main": 3, "bwd_dqdr": 5, "bwd_dkdudv": 3}
@@ -373,6 +391,7 @@ def main():
         timing["autograd_op_ms"] = time_events(autograd_step, min(args.steps, 100))
 
     kt = kernel_timings(w, ins)
+    mfma_loop = measured_mfma_peak_tflops(dev)
     dom = max(CREDIT, key=lambda k: kt.get(k, 0.0))
     ach = CREDIT[dom] * f1(w) / (kt[dom] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
@@ -391,6 +410,8 @@ def main():
         "config": {"workload": f"{args.workload}: {w['label']}", "credited_flops_per_step": flops,
                    "flop_convention": "11*F1 fwd+bwd (3 fwd + 8 bwd), F1=2*T*H*E*d_e*d_h"},
         "frac_of_mfma_peak": tflops / PEAK_BF16_TFLOPS,
+        "measured_mfma_loop_tflops": mfma_loop,
+        "frac_of_measured_mfma_loop": tflops / mfma_loop,
         "tokens_per_s": tokens / (ms * 1e-3),
         "peak_hbm_bytes": {"beyond_inputs": int(peak_extra), "inputs": int(base_mem),
                            "forbidden_intermediate_bytes_one_tensor": tokens * w["H"] * w["E"] * w["d_e"] * 2},

@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "_lib")
 LIB = os.path.join(LIBDIR, "libmhffn_hip.so")
-SOURCES = ["mhffn_capi.hip", "mhffn_fwd.hip", "mhffn_bwd.hip", "mhffn_f32.hip", "mhffn_gate.hip"]
+SOURCES = ["mhffn_capi.hip", "mhffn_fwd.hip", "mhffn_bwd.hip", "mhffn_f32.hip", "mhffn_gate.hip", "mhffn_probe.hip"]
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
     # packed fp32 VALU ops are kept out of the generated code on this hardware pool

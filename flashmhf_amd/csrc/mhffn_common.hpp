@@ -296,4 +296,7 @@ hipError_t launch_gate_fwd(const void* X, const float* Wn, float eps, const floa
 hipError_t launch_gate_bwd(const void* X, const float* Wn, float eps, const float* Wr, const void* dQ, int dq_tokmaj,
                            const float* dR, void* dX, float* dWn, float* dWr, const Dims& d, hipStream_t st);
 
+// Diagnostic (mhffn_probe.hip): register-resident MFMA loop.
+hipError_t launch_mfma_peak_probe(float* sink, int blocks, int iters, hipStream_t st);
+
 }  // namespace mhffn

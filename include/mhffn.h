@@ -153,6 +153,12 @@ int mhffn_gate_bwd(const void* X, const float* norm_weight, float eps, const flo
                    const void* dQ, int dq_token_layout, const float* dR,
                    void* dX, float* d_norm_weight, float* d_router, const mhffn_dims* dims, void* stream);
 
+/* Diagnostic, no counterpart in the reference: enqueues a register-resident loop of the matrix instruction the kernels use
+ * (`blocks` workgroups of four waves, `iters` x 32 instructions per wave, no memory traffic) and writes the number of
+ * floating-point operations it executes to *flops (host memory).  Timing it gives the rate the matrix cores sustain at
+ * the clock the device holds under load; bench.py reports it beside the nominal peak.  `sink` is one device float. */
+int mhffn_probe_mfma_peak(float* sink, int blocks, int iters, void* stream, double* flops);
+
 #ifdef __cplusplus
 }
 #endif
