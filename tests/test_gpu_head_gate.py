@@ -146,3 +146,37 @@ def test_layer_with_and_without_the_fused_prologue_agree():
     for name, a, b in zip(("y", "dx", "d_router", "d_q_norm", "d_w_self"), *outs):
         scale = max(b.abs().max().item(), 1e-6)
         assert (a - b).abs().max().item() <= 3e-2 * scale, (name, (a - b).abs().max().item(), scale)
+
+
+def test_gate_saturation_and_zero_rows():
+    """Zero rows (rsqrt of eps alone), logits far beyond the sigmoid's range in both directions, and a head whose every
+    logit underflows (sum of sigmoids below the clamp): forward and backward stay finite and on the oracle."""
+    from flashmhf_amd.head_gate import head_norm_gate
+    B, S, H, dh, E = 1, 64, 3, 128, 6
+    x, w, router = _inputs(B, S, H, dh, E, True, seed=9)
+    x[:, 3] = 0                                   # a token whose every head row is zero
+    router = router.float()
+    router[0] *= 400.0                            # head 0: logits of a few hundred, both signs
+    router[1] = -3.0 * w[1].float().sign().unsqueeze(-1) * torch.ones(dh, E)   # head 1: strongly negative for most rows
+    router = router.bfloat16()
+    g = torch.Generator().manual_seed(10)
+    dQ = torch.randn(B, H, S, dh, generator=g).bfloat16()
+    dR = torch.randn(B, H, S, E, generator=g)
+    leaves = [x.float().requires_grad_(True), w.float().requires_grad_(True), router.float().requires_grad_(True)]
+    rq, rR = orc.head_norm_gate(leaves[0], leaves[1], leaves[2], eps=1e-6)
+    (rq * dQ.float()).sum().add((rR * dR).sum()).backward()
+    dev = "cuda:0"
+    xd, wd, rd = (t.to(dev).requires_grad_(True) for t in (x, w, router))
+    Q, R = head_norm_gate(xd, wd, rd, 1e-6)
+    torch.autograd.backward([Q, R], [dQ.to(dev), dR.to(dev)])
+    torch.cuda.synchronize()
+    assert torch.equal(Q[:, :, 3].cpu().float(), torch.zeros(B, H, dh))
+    torch.testing.assert_close(R[:, :, 3].cpu(), torch.full((B, H, E), 1.0 / E))
+    _, ref_R = orc.head_norm_gate(Q.detach().cpu().transpose(1, 2), None, router)
+    assert torch.isfinite(R).all()
+    torch.testing.assert_close(R.detach().cpu(), ref_R, rtol=1e-4, atol=1e-6)
+    for name, got, ref in (("dx", xd.grad, leaves[0].grad), ("d_router", rd.grad, leaves[2].grad),
+                           ("d_norm_weight", wd.grad, leaves[1].grad)):
+        assert torch.isfinite(got).all(), name
+        m = orc.error_metrics(got.float().cpu(), ref)
+        assert m["norm_max"] <= 2e-2 and m["mean_rel"] <= 2e-2, (name, m)
