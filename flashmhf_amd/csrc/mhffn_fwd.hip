@@ -33,8 +33,15 @@ struct FwdArgs {
     int tokmaj;           // Q, O token-major ([B, S, H, d_h]) instead of [B, H, S, d_h]
 };
 
-constexpr int FWD_NST = 4;                 // LDS stages (K | U | V tiles each)
-constexpr int FWD_STAGE_B = 3 * TILE_B;    // 24 KB
+// LDS ring of FWD_NST stages, laid out as three regions (all V tiles, all K tiles, all U tiles).  The block loop is
+// unrolled over the four stages, so the stage of every LDS access is a compile-time constant and goes into the
+// instruction's 16-bit offset field: the per-lane parts of the addresses (row, swizzled chunk) are computed once before the
+// loop and no step spends VALU instructions on addresses.  V and K regions lie below 64 KB; the U reads use a second set
+// of per-lane bases that already contains the U region's start.
+constexpr int FWD_NST = 4;
+constexpr int FWD_REGION_B = FWD_NST * TILE_B;   // 32 KB
+constexpr int FWD_V0 = 0, FWD_K0 = FWD_REGION_B, FWD_U0 = 2 * FWD_REGION_B;
+constexpr int FWD_RING_B = 3 * FWD_REGION_B;     // 96 KB
 
 template <int DH>
 __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
@@ -43,7 +50,7 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     constexpr int FILL = 24 / NW;
     constexpr int NG1 = 4 * KS, NG2 = 4 * CT, NSLOT = NG1 + NG2;   // MFMAs per step
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-    float* sR = reinterpret_cast<float*>(smem + FWD_NST * FWD_STAGE_B);   // [E][BT]
+    float* sR = reinterpret_cast<float*>(smem + FWD_RING_B);   // [E][BT]
 
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -57,21 +64,21 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     const bf16_t* Kh = p.K + wbase;
     const long offU = p.U - p.K, offV = p.V - p.K;
 
-    auto issue_block = [&](int blk) {
+    auto issue_block = [&](int blk, int stage) {
         const int bc = blk < nblk ? blk : nblk - 1;
-        unsigned char* st = smem + (blk % FWD_NST) * FWD_STAGE_B;
         const long roff = (long)bc * JB * DH;
 #pragma unroll
         for (int k = 0; k < FILL; ++k) {
             const int id = wave + NW * k;
             const int which = id >> 3;
             const long toff = which == 0 ? 0 : (which == 1 ? offU : offV);
-            tile_fill_ins<DH>(Kh + toff + roff, DH, st + which * TILE_B, id & 7, lane);
+            const int region = which == 0 ? FWD_K0 : (which == 1 ? FWD_U0 : FWD_V0);
+            tile_fill_ins<DH>(Kh + toff + roff, DH, smem + region + stage * TILE_B, id & 7, lane);
         }
     };
-    issue_block(0);
-    issue_block(1);
-    issue_block(2);
+    issue_block(0, 0);
+    issue_block(1, 1);
+    issue_block(2, 2);
 
     bf16x8 q[2][KS];
 #pragma unroll
@@ -98,19 +105,29 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
 
     const int krow = row_perm32(l32);
     const TrLane<CT> trl = make_tr_lane<CT, 8, 4>(lane);
+    // per-lane bases of the K and U row reads for every k-step (stage 0); the stage is added as an immediate
+    const unsigned char* kbase[KS];
+    const unsigned char* ubase[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        kbase[ks] = smem + FWD_K0 + krow * TILE_ROW_B + (((2 * ks + g) ^ swz16(krow)) << 4);
+        ubase[ks] = kbase[ks] + (FWD_U0 - FWD_K0);
+    }
+    const unsigned smem0 = lds_addr(smem);
 
-    // consumes M/N of block blk (mc, nc), produces M/N of block blk+1 (mn, nn)
-    auto step = [&](int blk, int e, f32x16 (&mc)[2], f32x16 (&nc)[2], f32x16 (&mn)[2], f32x16 (&nn)[2]) {
+    // consumes M/N of block blk (mc, nc), produces M/N of block blk+1 (mn, nn); ST = blk % FWD_NST
+    auto step = [&](auto st_, int blk, int e, f32x16 (&mc)[2], f32x16 (&nc)[2], f32x16 (&mn)[2], f32x16 (&nn)[2]) {
+        constexpr int ST = decltype(st_)::value, STN = (ST + 1) % FWD_NST;
         wait_vmcnt<FILL>();   // blocks <= blk+1 have landed (only block blk+2's loads may be in flight)
         __syncthreads();      // ... for every wave; and every wave is done with the stage about to be refilled
-        issue_block(blk + 3);
+        issue_block(blk + 3, (ST + 3) % FWD_NST);
 
         float r[2];
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct)
             r[ct] = blk < nblk ? sR[(e < p.E ? e : p.E - 1) * BT + wave * 64 + ct * 32 + l32] : 0.0f;
-        const unsigned char* st_next = smem + ((blk + 1) % FWD_NST) * FWD_STAGE_B;
-        const unsigned sV = lds_addr(smem + (blk % FWD_NST) * FWD_STAGE_B + 2 * TILE_B);
+        auto read_k = [&](int ks) { return *reinterpret_cast<const bf16x8*>(kbase[ks] + STN * TILE_B); };
+        auto read_u = [&](int ks) { return *reinterpret_cast<const bf16x8*>(ubase[ks] + STN * TILE_B); };
 
         // V^T operands of this block's second product first: these reads are issued from inline assembly, so the
         // compiler's own lgkmcnt bookkeeping for the K/U reads below does not know them; LDS returns in order, so any of
@@ -119,14 +136,14 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
         TrOperand av[CT][2];
 #pragma unroll
         for (int i = 0; i < CT; ++i) {
-            av[i][0] = tile_read_cols_async<0>(sV, trl, i);
-            av[i][1] = tile_read_cols_async<4096>(sV, trl, i);
+            av[i][0] = tile_read_cols_async<FWD_V0 + ST * TILE_B>(smem0, trl, i);
+            av[i][1] = tile_read_cols_async<FWD_V0 + ST * TILE_B + 4096>(smem0, trl, i);
         }
         bf16x8 ak[3], au[3];   // K/U operand ring, two k-steps ahead
-        ak[0] = tile_read_rows(st_next, krow, 0, g);
-        au[0] = tile_read_rows(st_next + TILE_B, krow, 0, g);
-        ak[1] = tile_read_rows(st_next, krow, 1, g);
-        au[1] = tile_read_rows(st_next + TILE_B, krow, 1, g);
+        ak[0] = read_k(0);
+        au[0] = read_u(0);
+        ak[1] = read_k(1);
+        au[1] = read_u(1);
         bf16x8 pt[2][2];
         float e0 = 0, e1 = 0, xn0 = 0, xn1 = 0;   // carried between the chunks of one element pair
         __builtin_amdgcn_sched_barrier(0);
@@ -156,8 +173,8 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
             if constexpr (k < NG1) {
                 constexpr int ks = k / 4, w = k % 4, ct = w >> 1;
                 if constexpr (w == 0 && ks + 2 < KS) {
-                    ak[(ks + 2) % 3] = tile_read_rows(st_next, krow, ks + 2, g);
-                    au[(ks + 2) % 3] = tile_read_rows(st_next + TILE_B, krow, ks + 2, g);
+                    ak[(ks + 2) % 3] = read_k(ks + 2);
+                    au[(ks + 2) % 3] = read_u(ks + 2);
                 }
                 if constexpr ((w & 1) == 0) {
                     if constexpr (ks == 0) mfma32_vgpr_first_bacc(mn[ct], ak[0], q[ct][0]);
@@ -187,10 +204,9 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     wait_vmcnt<2 * FILL>();   // block 0 (and the Q / R loads before it) have landed
     __syncthreads();
     {
-        const unsigned char* st = smem;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const bf16x8 a = tile_read_rows(st, krow, ks, g), u = tile_read_rows(st + TILE_B, krow, ks, g);
+            const bf16x8 a = *reinterpret_cast<const bf16x8*>(kbase[ks]), u = *reinterpret_cast<const bf16x8*>(ubase[ks]);
 #pragma unroll
             for (int ct = 0; ct < 2; ++ct) {
                 if (ks == 0) { mfma32_vgpr_first_bacc(mA[ct], a, q[ct][0]); mfma32_vgpr_first_bacc(nA[ct], u, q[ct][0]); }
@@ -200,12 +216,30 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
         mfma_result_fence(mA[0], nA[0], mA[1]);   // the element-wise code of step 0 reads these results
         mfma_result_fence(nA[1]);
     }
-    int e = 0, jb = 0;
-    for (int blk = 0; blk < nblk; blk += 2) {   // pairs: the two M/N register sets alternate; an odd count ends in a
-        step(blk, e, mA, nA, mB, nB);           // phantom block whose gate value is 0
+    // Four blocks per trip (one per LDS stage; the two M/N register sets alternate), then one last pair on stages 0, 1
+    // where the count leaves one or two blocks; an odd count ends in a phantom block whose gate value is 0.
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+    using S3 = std::integral_constant<int, 3>;
+    int e = 0, jb = 0, blk = 0;
+    auto advance = [&]() {
         if (++jb == p.nbe) { jb = 0; ++e; }
-        step(blk + 1, e, mB, nB, mA, nA);
-        if (++jb == p.nbe) { jb = 0; ++e; }
+    };
+    for (; blk + 2 < nblk; blk += 4) {
+        step(S0{}, blk, e, mA, nA, mB, nB);
+        advance();
+        step(S1{}, blk + 1, e, mB, nB, mA, nA);
+        advance();
+        step(S2{}, blk + 2, e, mA, nA, mB, nB);
+        advance();
+        step(S3{}, blk + 3, e, mB, nB, mA, nA);
+        advance();
+    }
+    if (blk < nblk) {
+        step(S0{}, blk, e, mA, nA, mB, nB);
+        advance();
+        step(S1{}, blk + 1, e, mB, nB, mA, nA);
     }
     wait_vmcnt<0>();      // drain the phantom prefetches before the workgroup's LDS is released
 
@@ -232,7 +266,7 @@ template <int DH>
 static hipError_t launch_fwd_t(const FwdArgs& a, const Dims& d, hipStream_t st)
 {
     const int tokw = 256;
-    const int smem = FWD_NST * FWD_STAGE_B + d.E * tokw * (int)sizeof(float);
+    const int smem = FWD_RING_B + d.E * tokw * (int)sizeof(float);
     if (smem > 160 * 1024) return hipErrorInvalidValue;
     static LdsOptIn optin;
     const hipError_t e = ensure_dynamic_lds(optin, (const void*)mhffn_fwd_kernel<DH>, smem);
