@@ -47,6 +47,10 @@ class RMSNorm(nn.Module):
         self.eps = eps
 
     def forward(self, x):
+        if self.weight.dim() == 1 and x.is_cuda:
+            # whole-row norm of the decoder blocks: torch's fused kernel (fp32 inside, one rounding at the end instead of
+            # the two of `weight * normed.to(dtype)`)
+            return F.rms_norm(x, (x.shape[-1],), self.weight.to(x.dtype), self.eps)
         xf = x.float()
         xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)
         if self.weight.dim() == 1:
@@ -122,17 +126,18 @@ class MHFFNLayer(nn.Module):
         return self.w_self_2(O.transpose(1, 2).reshape(B, S, hid))  # token-major O: the reshape is a view
 
 
-def _rotary(seq_len, head_dim, base, device):
+def _rotary(seq_len, head_dim, base, device, dtype):
+    """cos/sin tables [S, head_dim] in the activations' dtype (computed in fp32)."""
     inv = 1.0 / (base ** (torch.arange(0, head_dim, 2, device=device, dtype=torch.float32) / head_dim))
     ang = torch.outer(torch.arange(seq_len, device=device, dtype=torch.float32), inv)
     ang = torch.cat((ang, ang), dim=-1)
-    return ang.cos(), ang.sin()
+    return ang.cos().to(dtype), ang.sin().to(dtype)
 
 
 def _apply_rotary(x, cos, sin):
     half = x.shape[-1] // 2
     rot = torch.cat((-x[..., half:], x[..., :half]), dim=-1)
-    return (x.float() * cos + rot.float() * sin).to(x.dtype)
+    return x * cos + rot * sin
 
 
 class CausalSelfAttention(nn.Module):
@@ -142,10 +147,10 @@ class CausalSelfAttention(nn.Module):
         self.qkv = nn.Linear(hidden_size, 3 * hidden_size, bias=False)
         self.out = nn.Linear(hidden_size, hidden_size, bias=False)
 
-    def forward(self, x):
+    def forward(self, x, rope=None):
         B, S, hid = x.shape
         q, k, v = self.qkv(x).view(B, S, 3, self.num_heads, self.head_dim).permute(2, 0, 3, 1, 4)
-        cos, sin = _rotary(S, self.head_dim, self.rope_base, x.device)
+        cos, sin = rope if rope is not None else _rotary(S, self.head_dim, self.rope_base, x.device, x.dtype)
         q, k = _apply_rotary(q, cos, sin), _apply_rotary(k, cos, sin)
         y = F.scaled_dot_product_attention(q, k, v, is_causal=True)
         return self.out(y.transpose(1, 2).reshape(B, S, hid))
@@ -159,8 +164,8 @@ class MHFFNDecoderBlock(nn.Module):
         self.post_attn_norm = RMSNorm((hidden_size,), eps)
         self.mlp = MHFFNLayer(hidden_size, ffn_heads, num_experts, expert_dim, rms_norm_eps=eps, **layer_kw)
 
-    def forward(self, x):
-        x = x + self.attn(self.input_norm(x))
+    def forward(self, x, rope=None):
+        x = x + self.attn(self.input_norm(x), rope)
         return x + self.mlp(self.post_attn_norm(x))
 
 
@@ -181,8 +186,10 @@ class MHFFNDecoder(nn.Module):
 
     def forward(self, ids, labels=None):
         x = self.embed(ids)
+        attn = self.blocks[0].attn
+        rope = _rotary(ids.shape[1], attn.head_dim, attn.rope_base, x.device, x.dtype)   # one table for every block
         for blk in self.blocks:
-            x = blk(x)
+            x = blk(x, rope)
         logits = self.lm_head(self.norm(x))
         if labels is None:
             return logits
