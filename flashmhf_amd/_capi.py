@@ -15,12 +15,14 @@ LIB_PATH = os.path.join(_HERE, "_lib", "libmhffn_hip.so")
 
 DTYPE_BF16, DTYPE_F32 = 0, 1
 OK = 0
-ERR_NULL_POINTER, ERR_DTYPE, ERR_HEAD_DIM, ERR_EXPERT_DIM, ERR_SHAPE, ERR_WORKSPACE, ERR_LAUNCH, ERR_ALIGNMENT = range(-1, -9, -1)
+(ERR_NULL_POINTER, ERR_DTYPE, ERR_HEAD_DIM, ERR_EXPERT_DIM, ERR_SHAPE, ERR_WORKSPACE, ERR_LAUNCH, ERR_ALIGNMENT,
+ ERR_STATIC_SCRATCH) = range(-1, -10, -1)
+STATIC_SCRATCH_BYTES = 96 << 20
 
 EXPORTS = (
     "mhffn_strerror", "mhffn_is_supported", "mhffn_check_dims", "mhffn_fwd_workspace_bytes",
     "mhffn_bwd_workspace_bytes", "mhffn_fwd", "mhffn_bwd", "mhffn_fwd_phases", "mhffn_bwd_phases",
-    "mhffn_fwd_layout", "mhffn_bwd_layout", "mhffn_gate_fwd", "mhffn_gate_bwd",
+    "mhffn_fwd_layout", "mhffn_bwd_layout", "mhffn_bwd_static", "mhffn_gate_fwd", "mhffn_gate_bwd",
     "mhffn_probe_mfma_peak",
 )
 TOKENS_BHSD, TOKENS_BSHD = 0, 1     # layout of Q, O, dO, dQ
@@ -59,6 +61,7 @@ def lib():
         L.mhffn_fwd_layout.argtypes = [vp] * 6 + [vp, ctypes.c_size_t, dp, ctypes.c_int, ctypes.c_int, vp, ctypes.c_int]
         L.mhffn_bwd_layout.argtypes = ([vp] * 6 + [vp] * 5 + [ctypes.c_int, vp, ctypes.c_size_t, dp, ctypes.c_int,
                                                               ctypes.c_int, vp, ctypes.c_int])
+        L.mhffn_bwd_static.argtypes = [vp] * 6 + [vp] * 5 + [ctypes.c_int, dp, ctypes.c_int, ctypes.c_int, vp]
         L.mhffn_gate_fwd.argtypes = [vp, vp, ctypes.c_float, vp, vp, vp, dp, vp]
         L.mhffn_gate_bwd.argtypes = [vp, vp, ctypes.c_float, vp, vp, ctypes.c_int, vp, vp, vp, vp, dp, vp]
         L.mhffn_probe_mfma_peak.argtypes = [vp, ctypes.c_int, ctypes.c_int, vp, ctypes.POINTER(ctypes.c_double)]

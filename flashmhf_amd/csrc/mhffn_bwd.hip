@@ -568,7 +568,10 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
 }
 
 // ------------------------------------------------------------------------------------------------ host side
-static int pick_nslice(const Dims& d)
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// Token slices of the dK/dU/dV kernel for a workspace of `ws_bytes`: 0 if not even one slice of partials fits.
+static int pick_nslice(const Dims& d, size_t ws_bytes)
 {
     // Enough workgroups for ~2 per CU (256 CUs), but at least 8 token tiles per slice.
     const int nblk = d.E * (d.d_e / JB);
@@ -578,27 +581,28 @@ static int pick_nslice(const Dims& d)
     if (ns > ntile / 8) ns = ntile / 8;
     if (ns < 1) ns = 1;
     if (ns > 64) ns = 64;
+    const size_t slice_b = (size_t)3 * d.Hkuv * d.E * d.d_e * d.d_h * sizeof(float);
+    while (ns > 0 && align256((size_t)ns * slice_b) > ws_bytes) --ns;
     return (int)ns;
 }
-
-static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 size_t bwd_workspace_bytes_bf16(const Dims& d)
 {
     const size_t wsz = (size_t)d.Hkuv * d.E * d.d_e * d.d_h;
-    return align256((size_t)pick_nslice(d) * 3 * wsz * sizeof(float));
+    return align256((size_t)pick_nslice(d, ~(size_t)0) * 3 * wsz * sizeof(float));
+}
+
+size_t bwd_min_workspace_bytes_bf16(const Dims& d)
+{
+    return align256((size_t)3 * d.Hkuv * d.E * d.d_e * d.d_h * sizeof(float));
 }
 
 template <int DH>
 static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, const void* V, const float* R,
                                const void* dO, void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32,
-                               void* ws, const Dims& d, hipStream_t st, int phases)
+                               void* ws, size_t ws_bytes, const Dims& d, hipStream_t st, int phases)
 {
-#ifndef DQ_VARIANT
-#define DQ_VARIANT 1, 8
-#endif
-    constexpr int DQV[2] = {DQ_VARIANT};
-    constexpr int NCT = DQV[0], NW = DQV[1];
+    constexpr int NCT = 1, NW = 8;
     hipError_t err = hipSuccess;
     float* part = reinterpret_cast<float*>(ws);
     const int nbe = d.d_e / JB, G = d.H / d.Hkuv;
@@ -617,7 +621,8 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }
-    const int nslice = pick_nslice(d);
+    const int nslice = pick_nslice(d, ws_bytes);
+    if (nslice < 1) return hipErrorInvalidValue;
     if (phases & 4) {
         DwArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, part,
                  d.B, d.H, G, d.S, d.E, nbe, nslice, d.tokmaj};
@@ -650,13 +655,13 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
 }
 
 hipError_t launch_bwd_bf16(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
-                           void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32, void* ws, const Dims& d,
-                           hipStream_t st, int phases)
+                           void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32, void* ws, size_t ws_bytes,
+                           const Dims& d, hipStream_t st, int phases)
 {
     switch (d.d_h) {
-        case 64: return launch_bwd_t<64>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, d, st, phases);
-        case 96: return launch_bwd_t<96>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, d, st, phases);
-        case 128: return launch_bwd_t<128>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, d, st, phases);
+        case 64: return launch_bwd_t<64>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, ws_bytes, d, st, phases);
+        case 96: return launch_bwd_t<96>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, ws_bytes, d, st, phases);
+        case 128: return launch_bwd_t<128>(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_f32, ws, ws_bytes, d, st, phases);
     }
     return hipErrorInvalidValue;
 }

@@ -2,6 +2,11 @@
 #include "../../include/mhffn.h"
 #include "mhffn_common.hpp"
 
+// Scratch of mhffn_bwd_static: device memory that belongs to this code object, so the call needs no allocation.  Every
+// GPU the library is loaded on holds its own copy at its own address until the process ends.  In host code the array's
+// name is only a handle for hipGetSymbolAddress; kernels get the address that call returned, never the name.
+static __device__ __align__(256) unsigned char scratch[MHFFN_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -31,6 +36,25 @@ mhffn::Dims to_dims(const mhffn_dims* d, int token_layout = 0)
     return mhffn::Dims{d->B, d->H, d->Hkuv, d->S, d->d_h, d->E, d->d_e, token_layout};
 }
 
+std::atomic<void*> scratch_addr[mhffn::LDS_OPTIN_MAX_DEVICES];   // per device, looked up on the first call there
+
+hipError_t static_scratch_of_current_device(void** out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= mhffn::LDS_OPTIN_MAX_DEVICES) return hipErrorInvalidDevice;
+    void* p = scratch_addr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        scratch_addr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return hipSuccess;
+}
+
 }  // namespace
 
 extern "C" {
@@ -47,6 +71,8 @@ const char* mhffn_strerror(int code)
         case MHFFN_ERR_WORKSPACE: return "workspace missing or too small";
         case MHFFN_ERR_LAUNCH: return "kernel launch failed";
         case MHFFN_ERR_ALIGNMENT: return "pointer not 16-byte aligned";
+        case MHFFN_ERR_STATIC_SCRATCH:
+            return "problem too large for mhffn_bwd_static's fixed scratch (MHFFN_STATIC_SCRATCH_BYTES); use mhffn_bwd";
     }
     return "unknown error code";
 }
@@ -131,8 +157,37 @@ int mhffn_bwd_layout(const void* Q, const void* K, const void* U, const void* V,
                    ? MHFFN_OK
                    : MHFFN_ERR_LAUNCH;
     const hipError_t err = mhffn::launch_bwd_bf16(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR,
-                                                  grad_w_dtype == MHFFN_DTYPE_F32, workspace, d, (hipStream_t)stream,
-                                                  phases);
+                                                  grad_w_dtype == MHFFN_DTYPE_F32, workspace, need, d,
+                                                  (hipStream_t)stream, phases);
+    return err == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
+}
+
+int mhffn_bwd_static(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
+                     void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_dtype,
+                     const mhffn_dims* dims, int dtype, int token_layout, void* stream)
+{
+    const int rc = check_dims_impl(dims, dtype);
+    if (rc != MHFFN_OK) return rc;
+    if (token_layout != MHFFN_TOKENS_BHSD && token_layout != MHFFN_TOKENS_BSHD) return MHFFN_ERR_SHAPE;
+    if (grad_w_dtype != MHFFN_DTYPE_BF16 && grad_w_dtype != MHFFN_DTYPE_F32) return MHFFN_ERR_DTYPE;
+    if (!Q || !K || !U || !V || !R || !dO || !dQ || !dK || !dU || !dV || !dR) return MHFFN_ERR_NULL_POINTER;
+    const void* ptrs[] = {Q, K, U, V, R, dO, dQ, dK, dU, dV, dR};
+    for (const void* p : ptrs)
+        if (!aligned16(p)) return MHFFN_ERR_ALIGNMENT;
+    const mhffn::Dims d = to_dims(dims, token_layout);
+    // The float32 kernels take exactly the workspace they ask for; the bfloat16 launch uses fewer token slices when the
+    // array holds fewer partial sets than it would like, and needs room for one.
+    const size_t need = dtype == MHFFN_DTYPE_F32 ? mhffn::bwd_workspace_bytes_f32(d) : mhffn::bwd_min_workspace_bytes_bf16(d);
+    if (need > MHFFN_STATIC_SCRATCH_BYTES) return MHFFN_ERR_STATIC_SCRATCH;
+    void* ws = nullptr;
+    if (static_scratch_of_current_device(&ws) != hipSuccess) return MHFFN_ERR_LAUNCH;
+    hipError_t err;
+    if (dtype == MHFFN_DTYPE_F32)
+        err = mhffn::launch_bwd_f32(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_dtype == MHFFN_DTYPE_F32, ws, d,
+                                    (hipStream_t)stream, MHFFN_BWD_ALL);
+    else
+        err = mhffn::launch_bwd_bf16(Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, grad_w_dtype == MHFFN_DTYPE_F32, ws,
+                                     (size_t)MHFFN_STATIC_SCRATCH_BYTES, d, (hipStream_t)stream, MHFFN_BWD_ALL);
     return err == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
 }
 

@@ -275,12 +275,13 @@ __host__ __device__ inline TokRows tok_rows(int tokmaj, int b, int h, int H, int
 }
 
 size_t fwd_workspace_bytes_bf16(const Dims& d);
-size_t bwd_workspace_bytes_bf16(const Dims& d);
+size_t bwd_workspace_bytes_bf16(const Dims& d);       // what the launch uses when it may choose freely
+size_t bwd_min_workspace_bytes_bf16(const Dims& d);   // one token slice of partials: the least launch_bwd_bf16 accepts
 hipError_t launch_fwd_bf16(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
                            void* ws, const Dims& d, hipStream_t st, int phases);
 hipError_t launch_bwd_bf16(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,
                            void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32,
-                           void* ws, const Dims& d, hipStream_t st, int phases);
+                           void* ws, size_t ws_bytes, const Dims& d, hipStream_t st, int phases);
 
 // fp32 instantiation (mhffn_f32.hip): d_h a multiple of 8 up to 128, any d_e, any E.
 size_t bwd_workspace_bytes_f32(const Dims& d);

@@ -42,7 +42,8 @@ enum {
     MHFFN_ERR_SHAPE        = -5,  /* non-positive extent, H not a multiple of Hkuv, bf16 with E > 64 */
     MHFFN_ERR_WORKSPACE    = -6,  /* workspace missing or smaller than *_workspace_bytes() */
     MHFFN_ERR_LAUNCH       = -7,  /* hipGetLastError() after a launch */
-    MHFFN_ERR_ALIGNMENT    = -8   /* a tensor or workspace pointer is not 16-byte aligned */
+    MHFFN_ERR_ALIGNMENT    = -8,  /* a tensor or workspace pointer is not 16-byte aligned */
+    MHFFN_ERR_STATIC_SCRATCH = -9 /* mhffn_bwd_static only: the problem needs more than MHFFN_STATIC_SCRATCH_BYTES */
 };
 
 /* Problem extents, shared by every call. */
@@ -130,6 +131,27 @@ int mhffn_bwd_layout(const void* Q, const void* K, const void* U, const void* V,
                      int grad_w_dtype,
                      void* workspace, size_t workspace_bytes,
                      const mhffn_dims* dims, int dtype, int token_layout, void* stream, int phases);
+
+/* Backward for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc) and so have no workspace to hand to mhffn_bwd.  It has no counterpart in the reference, whose
+ * wrappers allocate with torch on every call (flash_mlp_moe.py:806-811, flash_ffn_moe_torch.py:17-21).
+ * Same arguments, kernels and results as mhffn_bwd_layout(..., MHFFN_BWD_ALL) without the workspace pair: the token-slice
+ * partial sums of dK, dU, dV live in a fixed array of MHFFN_STATIC_SCRATCH_BYTES that is part of the library's device
+ * code (each GPU the library runs on holds one copy until the process ends).  The call allocates nothing and frees
+ * nothing; its first call on a device looks the array's address up once.
+ *   - bfloat16: the dK/dU/dV kernel runs with as many token slices as fit the array (fewer than mhffn_bwd would use on
+ *     large problems: dK, dU, dV then differ from mhffn_bwd's in the last float32 bits of the partial sums' order, and
+ *     the kernel is slower), and needs room for one slice: 3 * Hkuv * E * d_e * d_h * 4 bytes.  Larger problems, and
+ *     float32 problems whose mhffn_bwd_workspace_bytes() exceed the array, return MHFFN_ERR_STATIC_SCRATCH before any
+ *     launch.
+ *   - all calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two threads) race.
+ *     Nothing in it has to start at zero (every element read was written by the same call), so it is never cleared. */
+#define MHFFN_STATIC_SCRATCH_BYTES (96u << 20)
+int mhffn_bwd_static(const void* Q, const void* K, const void* U, const void* V, const float* R,
+                     const void* dO,
+                     void* dQ, void* dK, void* dU, void* dV, float* dR,
+                     int grad_w_dtype,
+                     const mhffn_dims* dims, int dtype, int token_layout, void* stream);
 
 /* Head prologue of the block: what the caller does between its projection and the operator
  * (models/flashmhf/modeling_mhffnmoe.py:371-372 per-head RMSNorm, class at :97-135; :384-386 expert gate), in one pass
