@@ -117,8 +117,10 @@ def kernel_timings(w, ins, n=50):
 def measured_mfma_peak_tflops(dev):
     """Rate of a register-resident v_mfma_f32_32x32x16_bf16 loop on every SIMD (mhffn_probe_mfma_peak), ~5 ms per launch."""
     import ctypes
-    from flashmhf_amd import _capi
-    L = _capi.lib()
+    from flashmhf_amd import build as b
+    L = ctypes.CDLL(b.PROBE_LIB)
+    L.mhffn_probe_mfma_peak.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                        ctypes.POINTER(ctypes.c_double)]
     sink = torch.zeros(4, device=dev)
     flops = ctypes.c_double(0.0)
     blocks = torch.cuda.get_device_properties(dev).multi_processor_count
@@ -135,10 +137,97 @@ def measured_mfma_peak_tflops(dev):
 # Credited GEMMs per kernel (in units of F1): the forward's three; the dQ/dR kernel's recomputed M, N, dA and the two
 # dQ products; the dK/dU/dV kernel's three output products (its own recomputation of M, N, dA is not credited).
 CREDIT = {"fwd_main": 3, "bwd_dqdr": 5, "bwd_dkdudv": 3}
-# HBM bytes per launch at workload c2 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy
-# (profiles/c2_hbm_traffic_pmc.md); counters cannot be read from inside this process, so the figures are recorded here.
-TRAFFIC_C2 = {"fwd_main": 122.2e6, "bwd_dqdr": 160.5e6, "bwd_dkdudv": 334.4e6}
 HARDWARE = {"fwd_main": 3, "bwd_dqdr": 5, "bwd_dkdudv": 6}
+
+# HBM bytes per launch cannot be read from inside this process: they come from two rocprofv3 --pmc runs of this very
+# script (FETCH_SIZE, then WRITE_SIZE, with --calibrate-copy), which `--traffic-from` turns into a small JSON record
+# under profiles/ together with a hash of the kernel sources.  A run whose kernel sources hash differently reports
+# traffic null: the record no longer describes the kernels being timed.
+TRAFFIC_KERNELS = {"fwd_main": "mhffn_fwd_kernel", "bwd_dqdr": "mhffn_bwd_dqdr_kernel",
+                   "bwd_dkdudv": "mhffn_bwd_dkdudv_kernel", "bwd_reduce": "reduce_partials_kernel"}
+COPY_KERNEL, COPY_BYTES = "__amd_rocclr_copyBuffer", 256 << 20
+
+
+def traffic_record_path(workload):
+    return os.path.join(ROOT, "profiles", f"{workload}_hbm_traffic.json")
+
+
+def kernel_source_hash():
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "flashmhf_amd", "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".hpp")):
+            h.update(name.encode())
+            h.update(open(os.path.join(csrc, name), "rb").read())
+    return h.hexdigest()
+
+
+def write_traffic_record(workload, fetch_csv, write_csv, out_path):
+    """rocprofv3 counter CSVs (one FETCH_SIZE run, one WRITE_SIZE run of `bench.py --calibrate-copy`) -> JSON record.
+    Counter values are KiB per dispatch; each counter is scaled by what it reads for the 256 MiB device copy."""
+    import csv
+
+    def averages(path, counter):
+        acc = {}
+        with open(path, newline="") as f:
+            for r in csv.DictReader(f):
+                if r["Counter_Name"] == counter:
+                    acc.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
+        return {k: (sum(v) / len(v), len(v)) for k, v in acc.items()}
+
+    def pick(avgs, needle):
+        hits = [(v, n) for k, (v, n) in avgs.items() if needle in k]
+        if not hits:
+            raise SystemExit(f"no dispatch of {needle} in the counter file")
+        return max(hits, key=lambda x: x[1])
+
+    def copy_reading(path, counter):
+        # the runtime's copy kernel also moves the small input tensors: the 256 MiB calibration copies are its largest
+        # dispatches (four of them, equal to within counter noise)
+        vals = []
+        with open(path, newline="") as f:
+            for r in csv.DictReader(f):
+                if r["Counter_Name"] == counter and COPY_KERNEL in r["Kernel_Name"]:
+                    vals.append(float(r["Counter_Value"]))
+        big = [v for v in vals if v >= 0.9 * max(vals)] if vals else []
+        if len(big) < 2:
+            raise SystemExit("the calibration copies are missing: profile bench.py with --calibrate-copy")
+        return sum(big) / len(big)
+
+    fetch, write = averages(fetch_csv, "FETCH_SIZE"), averages(write_csv, "WRITE_SIZE")
+    f_scale = (COPY_BYTES / 1024.0) / copy_reading(fetch_csv, "FETCH_SIZE")
+    w_scale = (COPY_BYTES / 1024.0) / copy_reading(write_csv, "WRITE_SIZE")
+    rec = {"workload": workload, "kernel_source_sha256": kernel_source_hash(),
+           "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv -d <dir> -o p -- python3 bench.py "
+                      f"--workload {workload} --no-cpu --steps 2 --warmup 1 --calibrate-copy ; python3 bench.py --workload "
+                      f"{workload} --traffic-from <fetch csv> <write csv>",
+           "scale": {"FETCH_SIZE": f_scale, "WRITE_SIZE": w_scale,
+                     "reference": "256 MiB device copy (__amd_rocclr_copyBuffer) reads and writes 262144 KiB per launch"},
+           "kernels": {}}
+    for key, needle in TRAFFIC_KERNELS.items():
+        (fk, n), (wk, _) = pick(fetch, needle), pick(write, needle)
+        rec["kernels"][key] = {"launches": n, "fetch_bytes": fk * 1024 * f_scale, "write_bytes": wk * 1024 * w_scale,
+                               "hbm_bytes": fk * 1024 * f_scale + wk * 1024 * w_scale}
+    with open(out_path, "w") as f:
+        json.dump(rec, f, indent=1)
+        f.write("\n")
+    print(json.dumps(rec))
+
+
+def recorded_traffic(workload, kernel):
+    """(bytes per launch or None, note) for the dominant kernel from the committed counter record."""
+    path = traffic_record_path(workload)
+    if not os.path.exists(path):
+        return None, "no counter record for this workload under profiles/"
+    rec = json.load(open(path))
+    if rec.get("kernel_source_sha256") != kernel_source_hash():
+        return None, (f"profiles/{os.path.basename(path)} was measured on other kernel sources "
+                      f"({rec.get('kernel_source_sha256', '?')[:12]}); rerun the two rocprofv3 --pmc passes")
+    k = rec["kernels"].get(kernel)
+    if not k:
+        return None, f"kernel {kernel} not in profiles/{os.path.basename(path)}"
+    return k["hbm_bytes"], f"profiles/{os.path.basename(path)} (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, scaled by a 256 MiB copy)"
 
 
 def cpu_baseline(w, budget_s=25.0):
@@ -172,6 +261,47 @@ def cpu_baseline(w, budget_s=25.0):
     return {"value": flops / med / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "sample": f"oracle eager loop + autograd, fp32, B1xS{S} tokens of the same layer shape, median of {len(times)} runs, "
                       f"{med * 1e3:.1f} ms/step, tokens/s {B * S / med:.0f}"}
+
+
+def cpu_baseline_c0():
+    """The reference's CPU-runnable case: one 128M-config MH-FFN layer forward in fp32 through the layer wrapper
+    (Q = X W_q split into heads, R = sigmoid(X W_r) normalised over E, eager expert loop, W_o;
+    models/flashmhf/modeling_mhffnmoe.py:352-431) on X [2,128,768], H8 d_h96 E8 d_e256, seed 0;
+    all host threads, 3 warm-ups, 10 timed runs, median and min."""
+    import platform
+    from oracle import mhffn_oracle as orc
+    B, S, hid, H, E, de = 2, 128, 768, 8, 8, 256
+    dh = hid // H
+    g = torch.Generator().manual_seed(0)
+    X = torch.randn(B, S, hid, generator=g)
+    Wq, Wo = (torch.randn(hid, hid, generator=g) * hid ** -0.5 for _ in range(2))
+    Wr = torch.randn(hid, H * E, generator=g) * 0.02
+    K, U, V = (torch.randn(H, E, de, dh, generator=g) * dh ** -0.5 for _ in range(3))
+    run = lambda: orc.mhffn_layer_forward(X, Wq, Wr, K, U, V, Wo, num_heads=H, compute_dtype=torch.float32)
+    with torch.no_grad():
+        for _ in range(3):
+            run()
+        times = []
+        for _ in range(10):
+            t0 = time.perf_counter()
+            run()
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    flops = 3 * 2.0 * B * S * H * E * de * dh        # the fused path's three GEMMs; the two projections add 2*2*T*hid^2
+    model = platform.processor() or ""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {"value": flops / med / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "median_ms": med * 1e3, "min_ms": times[0] * 1e3, "tokens_per_s": B * S / med, "cpu_model": model,
+            "host_cpus": os.cpu_count(),
+            "sample": "oracle layer wrapper forward (Q = X W_q, sigmoid gate from X W_r, eager expert loop, W_o), fp32, "
+                      "B2xS128 hid 768 H8 d_h96 E8 d_e256, 3 warm-ups + 10 runs"}
 
 
 def swiglu_peak_bytes(tokens, hidden, inner, device):
@@ -320,7 +450,12 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy a few times (known-size reference for HBM traffic counters)")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: turn the counter_collection.csv files of two rocprofv3 --pmc runs of this script "
+                         "(FETCH_SIZE, WRITE_SIZE; both with --calibrate-copy) into profiles/<workload>_hbm_traffic.json")
     args = ap.parse_args()
+    if args.traffic_from:
+        return write_traffic_record(args.workload, args.traffic_from[0], args.traffic_from[1], traffic_record_path(args.workload))
     if args.gpus != 1:
         print("bench.py: this build runs the fused MH-FFN on ONE GPU; --gpus must be 1 "
               "(heads shard with no exchange and tokens with one all-reduce of dK, dU, dV, but no multi-GPU path is built)", file=sys.stderr)
@@ -394,8 +529,9 @@ def main():
     mfma_loop = measured_mfma_peak_tflops(dev)
     dom = max(CREDIT, key=lambda k: kt.get(k, 0.0))
     ach = CREDIT[dom] * f1(w) / (kt[dom] * 1e-3) / 1e12
+    traffic, traffic_note = recorded_traffic(args.workload, dom)
     roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": ach / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_C2.get(dom) if args.workload == "c2" else None,
+                "frac": ach / PEAK_BF16_TFLOPS, "traffic": traffic, "traffic_source": traffic_note,
                 "hardware_tflops": HARDWARE[dom] * f1(w) / (kt[dom] * 1e-3) / 1e12}
     kernels = {k: {"ms": v, **({"credited_tflops": CREDIT[k] * f1(w) / (v * 1e-3) / 1e12,
                                 "hardware_tflops": HARDWARE[k] * f1(w) / (v * 1e-3) / 1e12} if k in CREDIT else {})}
@@ -423,6 +559,7 @@ def main():
         out["swiglu_2048_5504_peak_hbm_bytes_beyond_inputs"] = swiglu_peak_bytes(tokens, 2048, 5504, dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(w)
+        out["cpu_baseline_c0"] = cpu_baseline_c0()
     print(json.dumps(out))
 
 

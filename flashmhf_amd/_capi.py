@@ -23,11 +23,10 @@ EXPORTS = (
     "mhffn_strerror", "mhffn_is_supported", "mhffn_check_dims", "mhffn_fwd_workspace_bytes",
     "mhffn_bwd_workspace_bytes", "mhffn_fwd", "mhffn_bwd", "mhffn_fwd_phases", "mhffn_bwd_phases",
     "mhffn_fwd_layout", "mhffn_bwd_layout", "mhffn_bwd_static", "mhffn_gate_fwd", "mhffn_gate_bwd",
-    "mhffn_probe_mfma_peak",
 )
 TOKENS_BHSD, TOKENS_BSHD = 0, 1     # layout of Q, O, dO, dQ
-FWD_PACK, FWD_MAIN, FWD_ALL = 1, 2, 3
-BWD_PACK, BWD_DQDR, BWD_DKDUDV, BWD_REDUCE, BWD_ALL = 1, 2, 4, 8, 15
+FWD_MAIN, FWD_ALL = 1, 1
+BWD_DQDR, BWD_DKDUDV, BWD_REDUCE, BWD_ALL = 1, 2, 4, 7
 
 
 class Dims(ctypes.Structure):
@@ -64,7 +63,6 @@ def lib():
         L.mhffn_bwd_static.argtypes = [vp] * 6 + [vp] * 5 + [ctypes.c_int, dp, ctypes.c_int, ctypes.c_int, vp]
         L.mhffn_gate_fwd.argtypes = [vp, vp, ctypes.c_float, vp, vp, vp, dp, vp]
         L.mhffn_gate_bwd.argtypes = [vp, vp, ctypes.c_float, vp, vp, ctypes.c_int, vp, vp, vp, vp, dp, vp]
-        L.mhffn_probe_mfma_peak.argtypes = [vp, ctypes.c_int, ctypes.c_int, vp, ctypes.POINTER(ctypes.c_double)]
         _lib = L
     return _lib
 

@@ -607,7 +607,7 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
     float* part = reinterpret_cast<float*>(ws);
     const int nbe = d.d_e / JB, G = d.H / d.Hkuv;
 
-    if (phases & 2) {
+    if (phases & PH_BWD_DQDR) {
         DqArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R,
                  (bf16_t*)dQ, dR, d.H, G, d.S, d.E, nbe, d.tokmaj};
         const int tokw = NW * 32 * NCT;
@@ -623,7 +623,7 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
     }
     const int nslice = pick_nslice(d, ws_bytes);
     if (nslice < 1) return hipErrorInvalidValue;
-    if (phases & 4) {
+    if (phases & PH_BWD_DKDUDV) {
         DwArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, part,
                  d.B, d.H, G, d.S, d.E, nbe, nslice, d.tokmaj};
         const int smem = DW_NST * DW_STAGE_B + 128;
@@ -640,7 +640,7 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }
-    if (phases & 8) {
+    if (phases & PH_BWD_REDUCE) {
         const long wsz = (long)d.Hkuv * d.E * d.d_e * d.d_h;
         const unsigned rblocks = (unsigned)((wsz / 4 + 255) / 256);
         if (grad_w_f32)

@@ -248,12 +248,4 @@ int mhffn_gate_bwd(const void* X, const float* norm_weight, float eps, const flo
                : MHFFN_ERR_LAUNCH;
 }
 
-int mhffn_probe_mfma_peak(float* sink, int blocks, int iters, void* stream, double* flops)
-{
-    if (!sink || !flops) return MHFFN_ERR_NULL_POINTER;
-    if (blocks <= 0 || iters <= 0 || blocks > (1 << 20)) return MHFFN_ERR_SHAPE;
-    *flops = 2.0 * 32 * 32 * 16 * 32.0 * (double)iters * 4.0 * (double)blocks;
-    return mhffn::launch_mfma_peak_probe(sink, blocks, iters, (hipStream_t)stream) == hipSuccess ? MHFFN_OK : MHFFN_ERR_LAUNCH;
-}
-
 }  // extern "C"

@@ -297,7 +297,7 @@ hipError_t launch_gate_fwd(const void* X, const float* Wn, float eps, const floa
 hipError_t launch_gate_bwd(const void* X, const float* Wn, float eps, const float* Wr, const void* dQ, int dq_tokmaj,
                            const float* dR, void* dX, float* dWn, float* dWr, const Dims& d, hipStream_t st);
 
-// Diagnostic (mhffn_probe.hip): register-resident MFMA loop.
-hipError_t launch_mfma_peak_probe(float* sink, int blocks, int iters, hipStream_t st);
+// Bits of the `phases` argument of the launch functions (the values of MHFFN_FWD_* / MHFFN_BWD_* in include/mhffn.h).
+constexpr int PH_FWD_MAIN = 1, PH_BWD_DQDR = 1, PH_BWD_DKDUDV = 2, PH_BWD_REDUCE = 4;
 
 }  // namespace mhffn

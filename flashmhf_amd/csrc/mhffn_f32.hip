@@ -310,21 +310,21 @@ hipError_t launch_bwd_f32(const void* Q, const void* K, const void* U, const voi
     if (e == hipSuccess) e = ensure_dynamic_lds(optin_dw, (const void*)dkdudv_f32_kernel, 128 * 1024);
     if (e != hipSuccess) return e;
     hipError_t err = hipSuccess;
-    if (phases & 2) {
+    if (phases & PH_BWD_DQDR) {
         const int smem = (5 * 32 * (d.d_h + 1) + 2 * TT * (JC + 1) + TT * 8) * (int)sizeof(float);
         dim3 grid((unsigned)d.H, (unsigned)((d.S + TT - 1) / TT), (unsigned)d.B);
         hipLaunchKernelGGL(dqdr_f32_kernel, grid, dim3(256), smem, st, a);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }
-    if (phases & 4) {
+    if (phases & PH_BWD_DKDUDV) {
         const int smem = (5 * 32 * (d.d_h + 1) + 3 * TT * (JC + 1)) * (int)sizeof(float);
         dim3 grid((unsigned)(d.E * ((d.d_e + JC - 1) / JC)), (unsigned)d.Hkuv, (unsigned)a.nslice);
         hipLaunchKernelGGL(dkdudv_f32_kernel, grid, dim3(256), smem, st, a);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }
-    if (phases & 8) {
+    if (phases & PH_BWD_REDUCE) {
         const long wsz = (long)d.Hkuv * d.E * d.d_e * d.d_h;
         const unsigned rblocks = (unsigned)((wsz + 255) / 256);
         if (grad_w_f32)

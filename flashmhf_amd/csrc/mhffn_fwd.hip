@@ -49,6 +49,10 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     constexpr int KS = DH / 16, CT = DH / 32, NW = 4, BT = NW * 64, NTHR = NW * 64;
     constexpr int FILL = 24 / NW;
     constexpr int NG1 = 4 * KS, NG2 = 4 * CT, NSLOT = NG1 + NG2;   // MFMAs per step
+    // The first products of a step are written by inline-assembly MFMAs whose results the next step's element-wise code
+    // reads without a fence of its own: the NG2 second-product MFMAs issued in between (32 matrix-pipe cycles each) are
+    // what covers the 18 wait states an MFMA result needs before a VALU read.
+    static_assert(NG2 >= 8, "the second-product MFMAs of a step must cover the hazard window of its first products");
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     float* sR = reinterpret_cast<float*>(smem + FWD_RING_B);   // [E][BT]
 
@@ -282,7 +286,7 @@ hipError_t launch_fwd_bf16(const void* Q, const void* K, const void* U, const vo
                            void* ws, const Dims& d, hipStream_t st, int phases)
 {
     (void)ws;
-    if (!(phases & 2)) return hipSuccess;
+    if (!(phases & PH_FWD_MAIN)) return hipSuccess;
     FwdArgs a{(const bf16_t*)Q, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, (bf16_t*)O,
               d.H,              d.H / d.Hkuv,     d.S,              d.E,              d.d_e / JB,
               d.tokmaj};

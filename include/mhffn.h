@@ -93,14 +93,13 @@ int mhffn_bwd(const void* Q, const void* K, const void* U, const void* V, const 
               const mhffn_dims* dims, int dtype, void* stream);
 
 /* Phase-selectable variants for profiling: run only the kernels whose bit is set in `phases`, on a workspace that an
- * earlier full call with the same arguments has filled.  The *_PACK bits are accepted and do nothing (the kernels
- * read K, U, V in place; there is no re-layout pass).  mhffn_fwd == mhffn_fwd_phases(..., MHFFN_FWD_ALL) and
+ * earlier full call with the same arguments has filled.  mhffn_fwd == mhffn_fwd_phases(..., MHFFN_FWD_ALL) and
  * mhffn_bwd == mhffn_bwd_phases(..., MHFFN_BWD_ALL).  They exist so a benchmark can bracket one kernel with HIP
  * events on the launch stream; the reference has no counterpart (its kernels are launched one per Python call,
  * flash_mlp_moe.py:832-866). */
 enum {
-    MHFFN_FWD_PACK = 1, MHFFN_FWD_MAIN = 2, MHFFN_FWD_ALL = 3,
-    MHFFN_BWD_PACK = 1, MHFFN_BWD_DQDR = 2, MHFFN_BWD_DKDUDV = 4, MHFFN_BWD_REDUCE = 8, MHFFN_BWD_ALL = 15
+    MHFFN_FWD_MAIN = 1, MHFFN_FWD_ALL = 1,
+    MHFFN_BWD_DQDR = 1, MHFFN_BWD_DKDUDV = 2, MHFFN_BWD_REDUCE = 4, MHFFN_BWD_ALL = 7
 };
 int mhffn_fwd_phases(const void* Q, const void* K, const void* U, const void* V, const float* R,
                      void* O, void* workspace, size_t workspace_bytes,
@@ -174,12 +173,6 @@ int mhffn_gate_fwd(const void* X, const float* norm_weight, float eps, const flo
 int mhffn_gate_bwd(const void* X, const float* norm_weight, float eps, const float* router,
                    const void* dQ, int dq_token_layout, const float* dR,
                    void* dX, float* d_norm_weight, float* d_router, const mhffn_dims* dims, void* stream);
-
-/* Diagnostic, no counterpart in the reference: enqueues a register-resident loop of the matrix instruction the kernels use
- * (`blocks` workgroups of four waves, `iters` x 32 instructions per wave, no memory traffic) and writes the number of
- * floating-point operations it executes to *flops (host memory).  Timing it gives the rate the matrix cores sustain at
- * the clock the device holds under load; bench.py reports it beside the nominal peak.  `sink` is one device float. */
-int mhffn_probe_mfma_peak(float* sink, int blocks, int iters, void* stream, double* flops);
 
 #ifdef __cplusplus
 }

@@ -14,7 +14,13 @@ Pinning status (what fixes each function independently of this file's own formul
   * mhffn_backward (analytic)-- torch.autograd of mhffn_forward in fp64, torch.autograd.gradcheck,
                                 central finite differences, and the scalar C backward.
   * tk_ground_truth          -- equals mhffn_forward up to rounding (same closed form).
-  * mhffn_layer_forward      -- library routines only (F.linear, sigmoid, sum).
+  * bf16_eager_autograd      -- torch.autograd of mhffn_forward (pinned above) on bf16 leaves; its gradients stay within
+                                the bf16 bar of the fp64 analytic backward on the reference script's shapes.
+  * router_gate              -- hand-computed rows (logits (0, ln 3) -> (0.4, 0.6), which a softmax misses by 0.15), the
+                                zero-router and all-saturated (clamp) cases, per-head routers with swapped experts.
+  * mhffn_layer_forward      -- an independent per-head, per-expert F.linear / torch.sigmoid / F.silu composition with
+                                E > 1 and a W_r whose columns all differ, so a swapped [H,E] view, a softmax gate or a
+                                transposed projection fails.
   * mhffn_block_forward      -- library routines around mhffn_forward; with E = 1 (gate identically 1) and no
                                 RMSNorm it equals F.linear -> per-head SwiGLU via F.linear -> F.linear; the per-head
                                 RMSNorm equals F.rms_norm over d_h times the per-head weight; and it agrees with the
@@ -124,6 +130,16 @@ def mhffn_autograd(Q, K, U, V, R, dO, *, compute_dtype=torch.float64):
     out = mhffn_forward(*leaves, compute_dtype=compute_dtype)
     grads = torch.autograd.grad(out, leaves, dO.to(out.dtype))
     return out.detach(), grads
+
+
+def bf16_eager_autograd(Q, K, U, V, R, dO):
+    """The gradients the reference's eager path itself produces in bf16: the expert loop of
+    models/flashmhf/modeling_mhffnmoe.py:412-431 on bf16 tensors (R fp32, fp32 sum over experts, bf16 result) under
+    torch.autograd.  Used only to show that the HIP backward is at least as close to the fp64 gradients as this is."""
+    leaves = [t.detach().to(torch.bfloat16).requires_grad_(True) for t in (Q, K, U, V)]
+    leaves.append(R.detach().to(torch.float32).requires_grad_(True))
+    out = mhffn_forward(*leaves, compute_dtype=torch.bfloat16, out_dtype=torch.bfloat16)
+    return torch.autograd.grad(out, leaves, dO.to(torch.bfloat16))
 
 
 def router_gate(Qh, router):

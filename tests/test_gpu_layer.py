@@ -116,3 +116,29 @@ def test_legacy_single_expert_operator_is_a_per_head_swiglu():
     _check(out, ref.detach(), "O")
     for name, a, b in zip(("dQ", "dK", "dU", "dV"), gl, lv):
         _check(a.grad, b.grad, name)
+
+
+def test_fused_block_norm_stays_within_the_second_rounding_of_the_reference_form():
+    """The decoder shell's whole-row RMSNorm takes torch's fused kernel on the GPU (fp32 inside, one rounding at the end);
+    the reference form rounds twice, `weight * normed.to(dtype)` (models/flashmhf/modeling_mhffnmoe.py:73-89).  With the
+    bf16 weight the decoder runs with, the two differ only by that extra rounding: never more than two bf16 ulps, and
+    for a weight of ones (no second product) never more than one."""
+    from flashmhf_amd.mhffn_layer import RMSNorm
+    torch.manual_seed(3)
+    hid = 1024
+    x = torch.randn(4, 37, hid, device="cuda:0").bfloat16()
+    norm = RMSNorm((hid,), eps=1e-6).to("cuda:0")
+    with torch.no_grad():
+        norm.weight.copy_(torch.rand(hid) + 0.5)
+    norm = norm.to(torch.bfloat16)                                   # as MHFFNDecoder(...).to(torch.bfloat16) leaves it
+    xf = x.float()
+    normed = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).to(x.dtype)
+    with torch.no_grad():
+        got, ref = norm(x), norm.weight * normed                     # fused branch / reference form
+        assert got.dtype == ref.dtype == torch.bfloat16
+        ulp = 2.0 ** (torch.floor(torch.log2(ref.float().abs().clamp(min=1e-30))) - 7)      # bf16: 8 significant bits
+        assert ((got.float() - ref.float()).abs() <= 2 * ulp).all()
+        assert (got != ref).float().mean().item() < 0.25
+        norm.weight.fill_(1.0)
+        ulp1 = 2.0 ** (torch.floor(torch.log2(normed.float().abs().clamp(min=1e-30))) - 7)
+        assert ((norm(x).float() - normed.float()).abs() <= ulp1).all()

@@ -26,8 +26,6 @@ def _token_major(t):
 @pytest.mark.parametrize("B,H,S,dh,E,de,Hk", CASES)
 def test_token_major_matches_contiguous_bit_for_bit(B, H, S, dh, E, de, Hk, dtype):
     from flashmhf_amd import mhffn_backward, mhffn_forward
-    if dtype == torch.float32 and S > 400:
-        pytest.skip("the fp32 instantiation is covered on the small cases")
     print(f"case B={B} H={H} S={S} dh={dh} E={E} de={de} Hk={Hk} {dtype}", flush=True)
     dev = "cuda:0"
     Q, K, U, V, R, dO = (t.to(dev) for t in make_inputs(B, H, S, dh, E, de, Hk, seed=31 + S, dtype=dtype))

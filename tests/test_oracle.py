@@ -151,6 +151,69 @@ def test_router_gate_rows_sum_to_one_and_layer_shapes():
     assert (Rg.sum(-1) - 1).abs().max().item() < 1e-6
 
 
+def test_router_gate_is_sigmoid_normalised_not_softmax_and_uses_each_heads_own_router():
+    """Hand-computed rows (models/flashmhf/modeling_mhffnmoe.py:384-386).  Logits (0, ln 3) give sigmoids (1/2, 3/4), so
+    R = (0.4, 0.6); a softmax would give (0.25, 0.75).  With a per-head router [H,d_h,E], head h must use router[h].
+    All-saturated negative logits give sigmoid = 0 in fp32, a zero sum clamped to 1e-20, and R = 0 without NaN."""
+    import math
+    ln3 = math.log(3.0)
+    router = torch.tensor([[0.0, ln3], [5.0, 7.0]])                       # [d_h=2, E=2]
+    Qh = torch.tensor([[1.0, 0.0], [0.0, 1.0]]).view(1, 1, 2, 2)          # token 0 selects row 0, token 1 row 1
+    R = orc.router_gate(Qh, router)
+    s5, s7 = 1 / (1 + math.exp(-5.0)), 1 / (1 + math.exp(-7.0))
+    want = torch.tensor([[0.4, 0.6], [s5 / (s5 + s7), s7 / (s5 + s7)]]).view(1, 1, 2, 2)
+    torch.testing.assert_close(R, want, rtol=1e-6, atol=1e-7)
+    soft = torch.softmax(Qh @ router, -1)
+    assert (R - soft).abs().max().item() > 0.1                             # the softmax reading is far away
+    # per-head routers: head 1's router has its expert columns swapped, so its gate rows must come out swapped
+    routers = torch.stack([router, router.flip(-1)])                       # [H=2, d_h, E]
+    R2 = orc.router_gate(Qh.expand(1, 2, 2, 2), routers)
+    torch.testing.assert_close(R2[:, 0], want[:, 0], rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(R2[:, 1], want[:, 0].flip(-1), rtol=1e-6, atol=1e-7)
+    # zero router: every expert gets exactly 1/E
+    assert torch.equal(orc.router_gate(torch.randn(1, 1, 3, 2), torch.zeros(2, 4)), torch.full((1, 1, 3, 4), 0.25))
+    # clamp branch: sigmoid(-200) underflows to 0 for every expert
+    Rz = orc.router_gate(torch.full((1, 1, 1, 2), 1.0), torch.full((2, 3), -100.0))
+    assert torch.equal(Rz, torch.zeros(1, 1, 1, 3))
+
+
+def test_layer_restatement_equals_an_independent_linear_sigmoid_composition():
+    """mhffn_layer_forward against F.linear / torch.sigmoid / F.silu written per head and per expert, with E > 1 and a
+    W_r whose columns all differ in scale, so that reading X W_r as [.., E, H] instead of [.., H, E], a softmax gate, a
+    transposed W_q or W_o, or a wrong head split of Q each change the result (modeling_mhffnmoe.py:352-431)."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(21)
+    B, S, hid, H, E, de = 2, 3, 12, 3, 2, 5
+    dh = hid // H
+    X = torch.randn(B, S, hid, generator=g, dtype=torch.float64)
+    Wq, Wo = (torch.randn(hid, hid, generator=g, dtype=torch.float64) / hid ** 0.5 for _ in range(2))
+    Wr = torch.randn(hid, H * E, generator=g, dtype=torch.float64) * torch.arange(1, H * E + 1, dtype=torch.float64) * 0.3
+    K, U, V = (torch.randn(H, E, de, dh, generator=g, dtype=torch.float64) for _ in range(3))
+    Y, Qh, R, Oh = orc.mhffn_layer_forward(X, Wq, Wr, K, U, V, Wo, num_heads=H, compute_dtype=torch.float64)
+
+    q_all = F.linear(X, Wq.t())                                   # x @ Wq
+    z_all = F.linear(X.float(), Wr.float().t())                   # the gate logits are fp32 in the reference (:384)
+    merged = torch.zeros(B, S, hid, dtype=torch.float64)
+    for h in range(H):
+        q = q_all[..., h * dh:(h + 1) * dh]
+        torch.testing.assert_close(Qh[:, h], q, rtol=1e-12, atol=1e-12)
+        sg = torch.sigmoid(z_all[..., h * E:(h + 1) * E])         # head h owns columns h*E .. h*E+E-1
+        r = sg / sg.sum(-1, keepdim=True)
+        torch.testing.assert_close(R[:, h], r, rtol=1e-6, atol=1e-7)
+        o = torch.zeros(B, S, dh, dtype=torch.float64)
+        for e in range(E):
+            a = F.silu(F.linear(q, K[h, e])) * F.linear(q, U[h, e])
+            o = o + F.linear(a, V[h, e].t()) * r[..., e:e + 1].double()
+        torch.testing.assert_close(Oh[:, h], o, rtol=1e-6, atol=1e-6)      # R is fp32 on both sides
+        merged[..., h * dh:(h + 1) * dh] = o
+    torch.testing.assert_close(Y, F.linear(merged, Wo.t()), rtol=1e-6, atol=1e-6)
+    # the mistakes this test is meant to catch do move the result
+    r_swapped = torch.sigmoid(z_all).view(B, S, E, H).permute(0, 3, 1, 2)
+    r_swapped = r_swapped / r_swapped.sum(-1, keepdim=True)
+    assert (r_swapped - R).abs().max().item() > 1e-2
+    assert (torch.softmax(z_all.view(B, S, H, E), -1).transpose(1, 2) - R).abs().max().item() > 1e-2
+
+
 def test_bf16_eager_is_within_tolerance_of_fp32_oracle():
     """The reference's own bf16 eager path vs the fp32 oracle on the same rounded inputs: documents that the
     2e-2 / 1e-2 bar is meaningful for the benchmark distributions."""
@@ -159,6 +222,25 @@ def test_bf16_eager_is_within_tolerance_of_fp32_oracle():
     got = orc.mhffn_forward(Q, K, U, V, R, compute_dtype=torch.bfloat16, out_dtype=torch.float32)
     m = orc.error_metrics(got, ref)
     assert m["max_abs"] < 2e-2 and m["mean_rel"] < 1e-2
+
+
+def test_bf16_eager_backward_error_on_the_reference_scripts_shapes():
+    """The reference's own bf16 eager backward against the fp64 analytic gradients on the shapes and distributions of
+    kernels/thunderkittens/run_from_python.py:6-12, 26-31 (every tensor N(0,1), loss (O*2).sum()): the error level the
+    HIP backward is held to on the GPU (tests/test_gpu_backward.py).  Raw max-abs errors are far above 2e-2 here because
+    the gradients themselves are of order 1e2..1e4; the scale-normalised figure is what the reference script prints."""
+    g = torch.Generator().manual_seed(77)
+    B, H, S, dh, E, de = 2, 4, 384, 128, 2, 128
+    Q = torch.randn(B, H, S, dh, generator=g).bfloat16()
+    K, U, V = (torch.randn(H, E, de, dh, generator=g).bfloat16() for _ in range(3))
+    R = torch.randn(B, H, S, E, generator=g)
+    dO = torch.full(Q.shape, 2.0).bfloat16()
+    ref = orc.mhffn_backward(Q, K, U, V, R, dO, compute_dtype=torch.float64)
+    eager = orc.bf16_eager_autograd(Q, K, U, V, R, dO)
+    for name, e, r in zip(("dQ", "dK", "dU", "dV", "dR"), eager, ref):
+        m = orc.error_metrics(e.float(), r)
+        print(name, m, "max|ref|", r.abs().max().item())
+        assert m["norm_max"] <= 5e-2 and m["mean_rel"] <= 2e-2, (name, m)
 
 
 def test_block_restatement_reduces_to_library_routines():
