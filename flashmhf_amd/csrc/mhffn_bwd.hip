@@ -303,29 +303,22 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         fill_coff[k] = c * 16;                        // bytes
     }
 
-    // Asynchronous fill of stage `sidx` with the tile under the cursor (nothing once all tiles are requested); every wave
-    // issues its share of LDS-direct loads (no staging registers), then the cursor advances.  Addresses are a
-    // wave-uniform 64-bit base plus a 32-bit lane offset.  Rows past the end of a sequence are clamped to its last row
-    // and their gate value is zeroed afterwards (zero_tail), which removes them from all three products.
-    // Returns the number of valid rows of the tile (32 unless it is a tail tile).
-    auto issue_tile = [&](int sidx) -> int {
-        const int last = p.S - pf_st * 32 - 1;                                       // last valid row of the tile (>= 0)
-        const char* qb = reinterpret_cast<const char*>(p.Q) + (long)pf_qrow * (DH * 2);
-        const char* gb = reinterpret_cast<const char*>(p.dO) + (long)pf_qrow * (DH * 2);
-        const char* rbp = reinterpret_cast<const char*>(p.R) + (long)pf_row * (p.E * 4);
-        unsigned char* sbase = smem_raw + sidx * DW_STAGE_B;
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            const int row = TAIL ? (fill_row[k] < last ? fill_row[k] : last) : fill_row[k];
-            const unsigned off = (unsigned)(row * qs * (DH * 2) + fill_coff[k]);
-            const int ins = wave + 4 * k;
-            __builtin_amdgcn_global_load_lds((gptr_t)(qb + off), (lptr_t)(sbase + ins * 1024), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gptr_t)(gb + off), (lptr_t)(sbase + TILE_B + ins * 1024), 16, 0, 0);
-        }
-        // gate values of this wave's expert for the 32 token rows (lanes 32..63 repeat them): one 4-byte element per lane
-        const int trow = TAIL ? (l32 < last ? l32 : last) : l32;
-        __builtin_amdgcn_global_load_lds((gptr_t)(rbp + (unsigned)((trow * p.E + e_w) * 4)),
-                                         (lptr_t)(sbase + 2 * TILE_B + wave * 256), 4, 0, 0);
+    // Asynchronous fill of a stage with the tile under the cursor (the last tile again once all are requested); every wave
+    // issues its share of LDS-direct loads (no staging registers).  Addresses are a wave-uniform 64-bit base plus a
+    // 32-bit lane offset.  Rows past the end of a sequence are clamped to its last row and their gate value is zeroed
+    // afterwards (zero_tail), which removes them from all three products.
+    // The work is split: prepare_tile computes the uniform bases of the tile under the cursor and advances the cursor
+    // (some forty scalar instructions; called under the last matrix instructions of a step, where the wave has issue
+    // slots to spare), fire_tile issues the loads (right behind the barrier) and returns the tile's valid rows.
+    const char* nx_qb = nullptr;
+    const char* nx_gb = nullptr;
+    const char* nx_rbp = nullptr;
+    int nx_last = 31;
+    auto prepare_tile = [&]() {
+        nx_last = p.S - pf_st * 32 - 1;                                       // last valid row of the tile (>= 0)
+        nx_qb = reinterpret_cast<const char*>(p.Q) + (long)pf_qrow * (DH * 2);
+        nx_gb = reinterpret_cast<const char*>(p.dO) + (long)pf_qrow * (DH * 2);
+        nx_rbp = reinterpret_cast<const char*>(p.R) + (long)pf_row * (p.E * 4);
         // advance unless this was the last tile of the slice (then later requests reload it, harmlessly)
         // (0/1 flags and multiplies: selects here were turned into branches inside the hot loop)
         const int more = pf_left > 1 ? 1 : 0;
@@ -336,6 +329,22 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         pf_qrow += more * 32 * qs + ws * (dqrow_s - 32 * qs) + wb * (dqrow_b - dqrow_s);
         pf_st = (pf_st + more) * (1 - ws);
         pf_bb = (pf_bb + ws) * (1 - wb);
+    };
+    auto fire_tile = [&](int sidx) -> int {
+        const int last = nx_last;
+        unsigned char* sbase = smem_raw + sidx * DW_STAGE_B;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int row = TAIL ? (fill_row[k] < last ? fill_row[k] : last) : fill_row[k];
+            const unsigned off = (unsigned)(row * qs * (DH * 2) + fill_coff[k]);
+            const int ins = wave + 4 * k;
+            __builtin_amdgcn_global_load_lds((gptr_t)(nx_qb + off), (lptr_t)(sbase + ins * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(nx_gb + off), (lptr_t)(sbase + TILE_B + ins * 1024), 16, 0, 0);
+        }
+        // gate values of this wave's expert for the 32 token rows (lanes 32..63 repeat them): one 4-byte element per lane
+        const int trow = TAIL ? (l32 < last ? l32 : last) : l32;
+        __builtin_amdgcn_global_load_lds((gptr_t)(nx_rbp + (unsigned)((trow * p.E + e_w) * 4)),
+                                         (lptr_t)(sbase + 2 * TILE_B + wave * 256), 4, 0, 0);
         return last + 1;
     };
     // Called by every wave after its own loads of stage `sidx` have landed and before the barrier that publishes
@@ -480,6 +489,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
                     __builtin_amdgcn_sched_barrier(0);
                 };
                 dk[ct] = mfma32(tr_value(tq[idx % 3]), dmB[s], dk[ct]);
+                if constexpr (idx == NSET - 1 && !TAIL) prepare_tile();     // scalar work of the next fill, under this MFMA
                 after_slot2(std::integral_constant<int, 3 * ct>{});
                 du[ct] = mfma32(tr_value(tq[idx % 3]), dnB[s], du[ct]);
                 after_slot2(std::integral_constant<int, 3 * ct + 1>{});
@@ -488,7 +498,12 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
             });
         }
         __builtin_amdgcn_sched_barrier(0);
-        mfma_result_fence(m, n, da);
+        // The first products were written by inline-assembly MFMAs the compiler cannot see.  The 6 CT contraction MFMAs
+        // issued since then cover the wait states before the next step's element-wise code reads them; what is still
+        // needed is that their registers stay allocated to the end of the step even when nothing reads them (the
+        // phantom steps), or the compiler hands them to other values that the late write would overwrite.
+        static_assert(6 * CT >= 8, "the contraction MFMAs of a step must cover the hazard window of its first products");
+        asm volatile("" :: "v"(m), "v"(n), "v"(da));
     };
 
     // Pipeline over tiles k = 0 .. nt (step k: first products of tile k, element-wise + contraction of tile k-1).
@@ -498,7 +513,11 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     f32x16 mA, nA, dA_, mB, nB, dB_;
 #pragma unroll
     for (int x = 0; x < 16; ++x) { mA[x] = 0.0f; nA[x] = 0.0f; dA_[x] = 0.0f; mB[x] = 0.0f; nB[x] = 0.0f; dB_[x] = 0.0f; }
-    int nv0 = issue_tile(0), nv1 = issue_tile(1), nv2 = 32, nv3 = 32;   // valid rows of the tile in each stage
+    prepare_tile();
+    int nv0 = fire_tile(0);
+    prepare_tile();
+    int nv1 = fire_tile(1), nv2 = 32, nv3 = 32;        // valid rows of the tile in each stage
+    if constexpr (!TAIL) prepare_tile();               // tile 2: fired behind the first barrier
     auto sync_step = [&](auto st_c, int nvalid, int& nv_next) {
         constexpr int ST = decltype(st_c)::value;
         // All of this wave's loads, not only the older tile's: a partial count (the next tile's loads still in flight)
@@ -507,8 +526,11 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         if constexpr (TAIL) {
             if (nvalid < 32) zero_tail(ST, nvalid);
         }
-        __syncthreads();
-        nv_next = issue_tile((ST + 2) % DW_NST);
+        // (a bare barrier: the LDS-direct loads were waited for just above, and this wave's LDS reads of the stage that
+        // is refilled next were consumed by the matrix instructions of the step before)
+        __builtin_amdgcn_s_barrier();
+        if constexpr (TAIL) prepare_tile();     // (the tail instantiation has no registers to spare for the early call)
+        nv_next = fire_tile((ST + 2) % DW_NST);
     };
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;

@@ -31,6 +31,7 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // 16-byte cop
 
 constexpr int JB = 32;          // rows of K/U/V per block
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr float FLT_MAX_F = 3.402823466e+38f;
 
 // MFMA output row rho (0..31) -> which row of the 32-row weight block must be fed as A-row rho so that
 // C registers 8s..8s+7 of lane group g hold j = 16s + 8g + kk.  rho = 8a + 4g + b  ->  16(a/2) + 8g + 4(a%2) + b.

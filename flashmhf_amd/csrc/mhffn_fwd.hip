@@ -126,10 +126,15 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
         __syncthreads();      // ... for every wave; and every wave is done with the stage about to be refilled
         issue_block(blk + 3, (ST + 3) % FWD_NST);
 
-        float r[2];
+        // The gate value enters through its reciprocal: r / (1 + e) = 1 / fma(e, 1/r, 1/r), one multiply fewer per
+        // element.  1/r is clamped to the largest finite float, so r = 0 (a zero gate, or the phantom block behind an odd
+        // count) makes the denominator at least FLT_MAX, whose reciprocal the hardware flushes to exactly 0.
+        float rinv[2];
 #pragma unroll
-        for (int ct = 0; ct < 2; ++ct)
-            r[ct] = blk < nblk ? sR[(e < p.E ? e : p.E - 1) * BT + wave * 64 + ct * 32 + l32] : 0.0f;
+        for (int ct = 0; ct < 2; ++ct) {
+            const float rv = blk < nblk ? sR[(e < p.E ? e : p.E - 1) * BT + wave * 64 + ct * 32 + l32] : 0.0f;
+            rinv[ct] = __builtin_amdgcn_fmed3f(__builtin_amdgcn_rcpf(rv), -FLT_MAX_F, FLT_MAX_F);
+        }
         auto read_k = [&](int ks) { return *reinterpret_cast<const bf16x8*>(kbase[ks] + STN * TILE_B); };
         auto read_u = [&](int ks) { return *reinterpret_cast<const bf16x8*>(ubase[ks] + STN * TILE_B); };
 
@@ -163,12 +168,12 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
                 e1 = __builtin_amdgcn_exp2f(-LOG2E * mc[ct][i1]);
                 xn0 = mc[ct][i0] * nc[ct][i0];
             } else if constexpr (third == 1) {
-                e0 = __builtin_amdgcn_rcpf(1.0f + e0);
-                e1 = __builtin_amdgcn_rcpf(1.0f + e1);
+                e0 = __builtin_amdgcn_rcpf(__builtin_fmaf(e0, rinv[ct], rinv[ct]));
+                e1 = __builtin_amdgcn_rcpf(__builtin_fmaf(e1, rinv[ct], rinv[ct]));
                 xn1 = mc[ct][i1] * nc[ct][i1];
             } else {
-                pt[ct][i0 >> 3][i0 & 7] = (bf16_t)(xn0 * (r[ct] * e0));
-                pt[ct][i0 >> 3][i1 & 7] = (bf16_t)(xn1 * (r[ct] * e1));
+                pt[ct][i0 >> 3][i0 & 7] = (bf16_t)(xn0 * e0);
+                pt[ct][i0 >> 3][i1 & 7] = (bf16_t)(xn1 * e1);
             }
         };
 
@@ -202,6 +207,10 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
             });
             __builtin_amdgcn_sched_barrier(0);
         });
+        // The first products are written by the matrix pipe long after their instruction has issued.  Keep their
+        // registers allocated to the end of the step even when nothing reads them (the phantom block behind an odd
+        // count): otherwise the compiler hands them to other values, which the late write then overwrites.
+        asm volatile("" :: "v"(mn[0]), "v"(mn[1]), "v"(nn[0]), "v"(nn[1]));
     };
 
     f32x16 mA[2], nA[2], mB[2], nB[2];
