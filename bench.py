@@ -80,7 +80,7 @@ def time_events(fn, n, warm=10):
     return a.elapsed_time(b) / n
 
 
-def kernel_timings(w, ins, n=50):
+def kernel_timings(w, ins, n=50, sample_state=True):
     """Average duration of each kernel, bracketed by events on the launch stream (torch's current stream)."""
     from flashmhf_amd import _capi
     Q, K, U, V, R, dO = ins
@@ -105,12 +105,64 @@ def kernel_timings(w, ins, n=50):
         assert rc == 0, rc
 
     fwd(_capi.FWD_ALL)
-    out = {"fwd_main": time_events(lambda: fwd(_capi.FWD_MAIN), n)}
+    runs = {"fwd_main": lambda: fwd(_capi.FWD_MAIN)}
     if "bwd" in w["passes"]:
         bwd(_capi.BWD_ALL)
-        out["bwd_dqdr"] = time_events(lambda: bwd(_capi.BWD_DQDR), n)
-        out["bwd_dkdudv"] = time_events(lambda: bwd(_capi.BWD_DKDUDV), n)
-        out["bwd_reduce"] = time_events(lambda: bwd(_capi.BWD_REDUCE), n)
+        runs.update(bwd_dqdr=lambda: bwd(_capi.BWD_DQDR), bwd_dkdudv=lambda: bwd(_capi.BWD_DKDUDV),
+                    bwd_reduce=lambda: bwd(_capi.BWD_REDUCE))
+    out = {k: time_events(f, n) for k, f in runs.items()}
+    state = {k: device_state_under(f) for k, f in runs.items() if k != "bwd_reduce"} if sample_state else {}
+    return out, state
+
+
+def device_state_under(fn, seconds=0.5):
+    """Shader clock (MHz) and package power (W) as the driver reports them (sysfs pp_dpm_sclk, hwmon power1_input)
+    while `fn` is launched back to back for `seconds`: median of the samples taken after the first 100 ms.  The clock a
+    kernel is given depends on the kernel: under matrix-heavy load the package sits at its power limit and the clock
+    settles well below the 2.4 GHz the nominal peak is quoted at.  Returns None where the files cannot be read."""
+    import glob
+    import threading
+    sclk = glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")
+    pwr = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")
+    cap = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap")
+    if not sclk:
+        return None
+    samples, stop = [], threading.Event()
+
+    def read_mhz():
+        for line in open(sclk[0]):
+            if line.rstrip().endswith("*"):
+                return float(line.split(":")[1].strip().split("M")[0])
+        return None
+
+    def sampler():
+        t0 = time.perf_counter()
+        while not stop.is_set():
+            try:
+                mhz = read_mhz()
+                w = float(open(pwr[0]).read()) / 1e6 if pwr else None
+                if time.perf_counter() - t0 > 0.1:
+                    samples.append((mhz, w))
+            except (OSError, ValueError, IndexError):
+                pass
+            time.sleep(0.004)
+
+    th = threading.Thread(target=sampler, daemon=True)
+    th.start()
+    t_end = time.perf_counter() + seconds
+    while time.perf_counter() < t_end:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+    stop.set()
+    th.join()
+    med = lambda xs: sorted(xs)[len(xs) // 2] if xs else None
+    out = {"sclk_mhz": med([m for m, _ in samples if m]), "power_w": med([w for _, w in samples if w]),
+           "samples": len(samples)}
+    try:
+        out["power_cap_w"] = float(open(cap[0]).read()) / 1e6 if cap else None
+    except (OSError, ValueError):
+        out["power_cap_w"] = None
     return out
 
 
@@ -131,7 +183,7 @@ def measured_mfma_peak_tflops(dev):
         assert rc == 0, rc
 
     ms = time_events(run, 5, warm=3)
-    return flops.value / (ms * 1e-3) / 1e12
+    return flops.value / (ms * 1e-3) / 1e12, device_state_under(run, seconds=0.4)
 
 
 # Credited GEMMs per kernel (in units of F1): the forward's three; the dQ/dR kernel's recomputed M, N, dA and the two
@@ -525,8 +577,8 @@ def main():
 
         timing["autograd_op_ms"] = time_events(autograd_step, min(args.steps, 100))
 
-    kt = kernel_timings(w, ins)
-    mfma_loop = measured_mfma_peak_tflops(dev)
+    kt, kstate = kernel_timings(w, ins)
+    mfma_loop, probe_state = measured_mfma_peak_tflops(dev)
     dom = max(CREDIT, key=lambda k: kt.get(k, 0.0))
     ach = CREDIT[dom] * f1(w) / (kt[dom] * 1e-3) / 1e12
     traffic, traffic_note = recorded_traffic(args.workload, dom)
@@ -534,7 +586,8 @@ def main():
                 "frac": ach / PEAK_BF16_TFLOPS, "traffic": traffic, "traffic_source": traffic_note,
                 "hardware_tflops": HARDWARE[dom] * f1(w) / (kt[dom] * 1e-3) / 1e12}
     kernels = {k: {"ms": v, **({"credited_tflops": CREDIT[k] * f1(w) / (v * 1e-3) / 1e12,
-                                "hardware_tflops": HARDWARE[k] * f1(w) / (v * 1e-3) / 1e12} if k in CREDIT else {})}
+                                "hardware_tflops": HARDWARE[k] * f1(w) / (v * 1e-3) / 1e12} if k in CREDIT else {}),
+                   **({"under_load": kstate[k]} if kstate.get(k) else {})}
                for k, v in kt.items()}
 
     out = {
@@ -547,6 +600,8 @@ def main():
                    "flop_convention": "11*F1 fwd+bwd (3 fwd + 8 bwd), F1=2*T*H*E*d_e*d_h"},
         "frac_of_mfma_peak": tflops / PEAK_BF16_TFLOPS,
         "measured_mfma_loop_tflops": mfma_loop,
+        "measured_mfma_loop_under_load": probe_state,
+        "nominal_peak_clock_mhz": 2400,
         "frac_of_measured_mfma_loop": tflops / mfma_loop,
         "tokens_per_s": tokens / (ms * 1e-3),
         "peak_hbm_bytes": {"beyond_inputs": int(peak_extra), "inputs": int(base_mem),

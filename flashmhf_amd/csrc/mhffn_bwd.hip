@@ -35,11 +35,11 @@ struct DqArgs {
 constexpr int DQ_NST = 4;                  // LDS stages (K | U | V tiles each)
 constexpr int DQ_STAGE_B = 3 * TILE_B;
 
-template <int DH, int NCT, int NW>
-__global__ __launch_bounds__(NW * 64) void mhffn_bwd_dqdr_kernel(DqArgs p)
+template <int DH>
+__global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
 {
-    constexpr int KS = DH / 16, CT = DH / 32;
-    constexpr int BT = NW * 32 * NCT;
+    constexpr int KS = DH / 16, CT = DH / 32, NW = 8;
+    constexpr int BT = NW * 32;
     constexpr int NTHR = NW * 64;
     constexpr int FILL = 24 / NW;          // tile-fill wave-instructions per wave and block (3 tiles x 8 / NW waves)
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -51,7 +51,7 @@ __global__ __launch_bounds__(NW * 64) void mhffn_bwd_dqdr_kernel(DqArgs p)
     const int hk = h / p.G;
     const long rowbase = ((long)b * p.H + h) * p.S;          // rows of R, dR
     const TokRows qrows = tok_rows(p.tokmaj, b, h, p.H, p.S);   // rows of Q, dO, dQ
-    const int tok0 = tb * BT + wave * (32 * NCT);
+    const int tok0 = tb * BT + wave * 32;
     const int nblk = p.E * p.nbe;
     const bf16_t* Kh = p.K + (long)hk * nblk * JB * DH;
     const long offU = p.U - p.K, offV = p.V - p.K;
@@ -71,17 +71,16 @@ __global__ __launch_bounds__(NW * 64) void mhffn_bwd_dqdr_kernel(DqArgs p)
     issue_block(0);
     issue_block(1);
 
-    bf16x8 q[NCT][KS], go[NCT][KS];
-#pragma unroll
-    for (int ct = 0; ct < NCT; ++ct) {
-        int t = tok0 + ct * 32 + l32;
+    bf16x8 q[KS], go[KS];
+    {
+        int t = tok0 + l32;
         t = t < p.S ? t : p.S - 1;
         const bf16_t* qr = p.Q + (qrows.base + (long)t * qrows.stride) * DH + 8 * g;
         const bf16_t* gr = p.dO + (qrows.base + (long)t * qrows.stride) * DH + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            q[ct][ks] = *reinterpret_cast<const bf16x8*>(qr + ks * 16);
-            go[ct][ks] = *reinterpret_cast<const bf16x8*>(gr + ks * 16);
+            q[ks] = *reinterpret_cast<const bf16x8*>(qr + ks * 16);
+            go[ks] = *reinterpret_cast<const bf16x8*>(gr + ks * 16);
         }
     }
     for (int idx = tid; idx < BT * p.E; idx += NTHR) {
@@ -90,21 +89,17 @@ __global__ __launch_bounds__(NW * 64) void mhffn_bwd_dqdr_kernel(DqArgs p)
         sR[(idx % p.E) * BT + idx / p.E] = p.R[(rowbase + t) * p.E + idx % p.E];
     }
 
-    f32x16 dq[CT][NCT];
+    f32x16 dq[CT];
 #pragma unroll
     for (int i = 0; i < CT; ++i)
 #pragma unroll
-        for (int ct = 0; ct < NCT; ++ct)
-#pragma unroll
-            for (int x = 0; x < 16; ++x) dq[i][ct][x] = 0.0f;
+        for (int x = 0; x < 16; ++x) dq[i][x] = 0.0f;
 
     const int krow = row_perm32(l32);
     const TrLane<CT> trl = make_tr_lane<CT, 8, 4>(lane);
     int blk = 0;
     for (int e = 0; e < p.E; ++e) {
-        float dr[NCT];
-#pragma unroll
-        for (int ct = 0; ct < NCT; ++ct) dr[ct] = 0.0f;
+        float dr = 0.0f;
         for (int jb = 0; jb < p.nbe; ++jb, ++blk) {
             wait_vmcnt<FILL>();       // block blk has landed (block blk+1 may be in flight)
             __syncthreads();
@@ -113,45 +108,36 @@ __global__ __launch_bounds__(NW * 64) void mhffn_bwd_dqdr_kernel(DqArgs p)
             const unsigned char* sK = smem + (blk % DQ_NST) * DQ_STAGE_B;
             const unsigned char* sU = sK + TILE_B;
             const unsigned char* sV = sU + TILE_B;
-            float r[NCT];
-#pragma unroll
-            for (int ct = 0; ct < NCT; ++ct) r[ct] = sR[e * BT + wave * (32 * NCT) + ct * 32 + l32];
+            const float r = sR[e * BT + wave * 32 + l32];
 
-            f32x16 m[NCT], n[NCT], da[NCT];
+            f32x16 m, n, da;
 #pragma unroll
-            for (int ct = 0; ct < NCT; ++ct)
-#pragma unroll
-                for (int x = 0; x < 16; ++x) { m[ct][x] = 0.0f; n[ct][x] = 0.0f; da[ct][x] = 0.0f; }
+            for (int x = 0; x < 16; ++x) { m[x] = 0.0f; n[x] = 0.0f; da[x] = 0.0f; }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const bf16x8 ak = tile_read_rows(sK, krow, ks, g);
                 const bf16x8 au = tile_read_rows(sU, krow, ks, g);
                 const bf16x8 av = tile_read_rows(sV, krow, ks, g);
-#pragma unroll
-                for (int ct = 0; ct < NCT; ++ct) {
-                    m[ct] = mfma32(ak, q[ct][ks], m[ct]);
-                    n[ct] = mfma32(au, q[ct][ks], n[ct]);
-                    da[ct] = mfma32(av, go[ct][ks], da[ct]);
-                }
+                m = mfma32(ak, q[ks], m);
+                n = mfma32(au, q[ks], n);
+                da = mfma32(av, go[ks], da);
             }
 
-            bf16x8 dmt[NCT][2], dnt[NCT][2];
+            bf16x8 dmt[2], dnt[2];
 #pragma unroll
-            for (int ct = 0; ct < NCT; ++ct)
+            for (int s = 0; s < 2; ++s)
 #pragma unroll
-                for (int s = 0; s < 2; ++s)
-#pragma unroll
-                    for (int kk = 0; kk < 8; ++kk) {
-                        const int i = 8 * s + kk;
-                        const float x = m[ct][i], nn = n[ct][i], a = da[ct][i];
-                        const float sg = fast_sigmoid(x);
-                        const float sl = x * sg;                 // silu(m)
-                        const float as = a * sl;
-                        dr[ct] = __builtin_fmaf(as, nn, dr[ct]);
-                        const float w = __builtin_fmaf(sl, 1.0f - sg, sg);    // silu'(m)
-                        dnt[ct][s][kk] = (bf16_t)(r[ct] * as);
-                        dmt[ct][s][kk] = (bf16_t)((r[ct] * a) * (nn * w));
-                    }
+                for (int kk = 0; kk < 8; ++kk) {
+                    const int i = 8 * s + kk;
+                    const float x = m[i], nn = n[i], a = da[i];
+                    const float sg = fast_sigmoid(x);
+                    const float sl = x * sg;                 // silu(m)
+                    const float as = a * sl;
+                    dr = __builtin_fmaf(as, nn, dr);
+                    const float w = __builtin_fmaf(sl, 1.0f - sg, sg);    // silu'(m)
+                    dnt[s][kk] = (bf16_t)(r * as);
+                    dmt[s][kk] = (bf16_t)((r * a) * (nn * w));
+                }
 
             // second products: operand pairs (Kt, Ut) are requested two steps ahead of the MFMAs that consume them; the
             // region is fenced so that the partial LDS waits below count exactly these reads
@@ -173,28 +159,23 @@ __global__ __launch_bounds__(NW * 64) void mhffn_bwd_dqdr_kernel(DqArgs p)
                     if constexpr (idx + 2 < NSET) request(std::integral_constant<int, idx + 2>{});
                     constexpr int ahead = (NSET - 1 - idx) < 2 ? (NSET - 1 - idx) : 2;
                     lds_tr_wait_n<4 * ahead>(tk[idx % 3], tu[idx % 3]);
-#pragma unroll
-                    for (int ct = 0; ct < NCT; ++ct) {
-                        dq[i][ct] = mfma32(tr_value(tk[idx % 3]), dmt[ct][s], dq[i][ct]);
-                        dq[i][ct] = mfma32(tr_value(tu[idx % 3]), dnt[ct][s], dq[i][ct]);
-                    }
+                    dq[i] = mfma32(tr_value(tk[idx % 3]), dmt[s], dq[i]);
+                    dq[i] = mfma32(tr_value(tu[idx % 3]), dnt[s], dq[i]);
                 });
             }
             __builtin_amdgcn_sched_barrier(0);
         }
         // dR[t, e]: the two lane halves hold disjoint j rows of the same token column.
-#pragma unroll
-        for (int ct = 0; ct < NCT; ++ct) {
-            const float tot = dr[ct] + __shfl_xor(dr[ct], 32);
-            const int t = tok0 + ct * 32 + l32;
+        {
+            const float tot = dr + __shfl_xor(dr, 32);
+            const int t = tok0 + l32;
             if (g == 0 && t < p.S) p.dR[(rowbase + t) * p.E + e] = tot;
         }
     }
     wait_vmcnt<0>();   // drain the phantom prefetches before the workgroup's LDS is released
 
-#pragma unroll
-    for (int ct = 0; ct < NCT; ++ct) {
-        const int t = tok0 + ct * 32 + l32;
+    {
+        const int t = tok0 + l32;
         if (t < p.S) {
             bf16_t* orow = p.dQ + (qrows.base + (long)t * qrows.stride) * DH;
 #pragma unroll
@@ -203,7 +184,7 @@ __global__ __launch_bounds__(NW * 64) void mhffn_bwd_dqdr_kernel(DqArgs p)
                 for (int a = 0; a < 4; ++a) {
                     bf16x4 v;
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) v[x] = (bf16_t)dq[i][ct][4 * a + x];
+                    for (int x = 0; x < 4; ++x) v[x] = (bf16_t)dq[i][4 * a + x];
                     *reinterpret_cast<bf16x4*>(orow + 32 * i + 8 * a + 4 * g) = v;
                 }
         }
@@ -624,7 +605,6 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
                                const void* dO, void* dQ, void* dK, void* dU, void* dV, float* dR, int grad_w_f32,
                                void* ws, size_t ws_bytes, const Dims& d, hipStream_t st, int phases)
 {
-    constexpr int NCT = 1, NW = 8;
     hipError_t err = hipSuccess;
     float* part = reinterpret_cast<float*>(ws);
     const int nbe = d.d_e / JB, G = d.H / d.Hkuv;
@@ -632,14 +612,14 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
     if (phases & PH_BWD_DQDR) {
         DqArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R,
                  (bf16_t*)dQ, dR, d.H, G, d.S, d.E, nbe, d.tokmaj};
-        const int tokw = NW * 32 * NCT;
+        const int tokw = 256;
         const int smem = DQ_NST * DQ_STAGE_B + d.E * tokw * (int)sizeof(float);
         if (smem > 160 * 1024) return hipErrorInvalidValue;
         static LdsOptIn optin;
-        err = ensure_dynamic_lds(optin, (const void*)mhffn_bwd_dqdr_kernel<DH, NCT, NW>, smem);
+        err = ensure_dynamic_lds(optin, (const void*)mhffn_bwd_dqdr_kernel<DH>, smem);
         if (err != hipSuccess) return err;
         dim3 grid((unsigned)d.H, (unsigned)((d.S + tokw - 1) / tokw), (unsigned)d.B);
-        hipLaunchKernelGGL((mhffn_bwd_dqdr_kernel<DH, NCT, NW>), grid, dim3(NW * 64), smem, st, a);
+        hipLaunchKernelGGL((mhffn_bwd_dqdr_kernel<DH>), grid, dim3(512), smem, st, a);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }
