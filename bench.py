@@ -90,7 +90,8 @@ def kernel_timings(w, ins, n=50, sample_state=True):
     dK, dU, dV = (torch.empty_like(K) for _ in range(3))
     dR = torch.empty_like(R)
     wsf = torch.empty(max(16, L.mhffn_fwd_workspace_bytes(dims, 0)), dtype=torch.uint8, device=Q.device)
-    wsb = torch.empty(L.mhffn_bwd_workspace_bytes(dims, 0), dtype=torch.uint8, device=Q.device)
+    ws_bytes = L.mhffn_bwd_workspace_bytes(dims, 0)          # 0 where dK/dU/dV run as one token slice (no reduce pass)
+    wsb = torch.empty(max(16, ws_bytes), dtype=torch.uint8, device=Q.device)
     st = torch.cuda.current_stream().cuda_stream
 
     def fwd(ph):
@@ -108,8 +109,9 @@ def kernel_timings(w, ins, n=50, sample_state=True):
     runs = {"fwd_main": lambda: fwd(_capi.FWD_MAIN)}
     if "bwd" in w["passes"]:
         bwd(_capi.BWD_ALL)
-        runs.update(bwd_dqdr=lambda: bwd(_capi.BWD_DQDR), bwd_dkdudv=lambda: bwd(_capi.BWD_DKDUDV),
-                    bwd_reduce=lambda: bwd(_capi.BWD_REDUCE))
+        runs.update(bwd_dqdr=lambda: bwd(_capi.BWD_DQDR), bwd_dkdudv=lambda: bwd(_capi.BWD_DKDUDV))
+        if ws_bytes:
+            runs.update(bwd_reduce=lambda: bwd(_capi.BWD_REDUCE))
     out = {k: time_events(f, n) for k, f in runs.items()}
     state = {k: device_state_under(f) for k, f in runs.items() if k != "bwd_reduce"} if sample_state else {}
     return out, state
@@ -258,6 +260,8 @@ def write_traffic_record(workload, fetch_csv, write_csv, out_path):
                      "reference": "256 MiB device copy (__amd_rocclr_copyBuffer) reads and writes 262144 KiB per launch"},
            "kernels": {}}
     for key, needle in TRAFFIC_KERNELS.items():
+        if key == "bwd_reduce" and not any(needle in k for k in fetch):
+            continue                                   # one token slice: dK/dU/dV are written by the kernel itself
         (fk, n), (wk, _) = pick(fetch, needle), pick(write, needle)
         rec["kernels"][key] = {"launches": n, "fetch_bytes": fk * 1024 * f_scale, "write_bytes": wk * 1024 * w_scale,
                                "hbm_bytes": fk * 1024 * f_scale + wk * 1024 * w_scale}

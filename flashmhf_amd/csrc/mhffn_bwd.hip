@@ -199,7 +199,9 @@ struct DwArgs {
     const bf16_t* U;
     const bf16_t* V;
     const float* R;
-    float* part;        // [nslice][3][Hkuv][E*d_e][DH] fp32 partial sums
+    float* part;        // [nslice][3][Hkuv][E*d_e][DH] fp32 partial sums (nslice > 1)
+    void* out[3];       // dK, dU, dV: written directly when there is one token slice
+    int out_f32;        // element type of out: 1 = float32, 0 = bfloat16
     int B, H, G, S, E, nbe, nslice;
     int tokmaj;         // Q, dO token-major ([B, S, H, d_h]) instead of [B, H, S, d_h]
 };
@@ -532,21 +534,53 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     wait_vmcnt<0>();
 
     if (active) {
-        // dK^T registers 4a+b of row tile ct: c = 32ct + 8a + 4g + b, column j = l32 -> 16-byte runs along c.
+        // dK^T registers 4a+b of row tile ct: c = 32ct + 8a + 4g + b, column j = l32 -> runs of 4 along c.
         const long wsz = (long)gridDim.x * nblk * JB * DH;   // elements of one weight tensor
-        float* base = p.part + (long)z * 3 * wsz + wrow * DH;
+        if (p.nslice > 1) {                                  // fp32 partial sums of this token slice
+            float* base = p.part + (long)z * 3 * wsz + wrow * DH;
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
+            for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
-            for (int a = 0; a < 4; ++a) {
-                const int c = 32 * ct + 8 * a + 4 * g;
-                f32x4 v0, v1, v2;
+                for (int a = 0; a < 4; ++a) {
+                    const int c = 32 * ct + 8 * a + 4 * g;
+                    f32x4 v0, v1, v2;
 #pragma unroll
-                for (int x = 0; x < 4; ++x) { v0[x] = dk[ct][4 * a + x]; v1[x] = du[ct][4 * a + x]; v2[x] = dv[ct][4 * a + x]; }
-                *reinterpret_cast<f32x4*>(base + c) = v0;
-                *reinterpret_cast<f32x4*>(base + wsz + c) = v1;
-                *reinterpret_cast<f32x4*>(base + 2 * wsz + c) = v2;
-            }
+                    for (int x = 0; x < 4; ++x) { v0[x] = dk[ct][4 * a + x]; v1[x] = du[ct][4 * a + x]; v2[x] = dv[ct][4 * a + x]; }
+                    *reinterpret_cast<f32x4*>(base + c) = v0;
+                    *reinterpret_cast<f32x4*>(base + wsz + c) = v1;
+                    *reinterpret_cast<f32x4*>(base + 2 * wsz + c) = v2;
+                }
+        } else if (p.out_f32) {                              // one slice: the sums are the gradients
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    const long o = wrow * DH + 32 * ct + 8 * a + 4 * g;
+                    f32x4 v0, v1, v2;
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) { v0[x] = dk[ct][4 * a + x]; v1[x] = du[ct][4 * a + x]; v2[x] = dv[ct][4 * a + x]; }
+                    *reinterpret_cast<f32x4*>(static_cast<float*>(p.out[0]) + o) = v0;
+                    *reinterpret_cast<f32x4*>(static_cast<float*>(p.out[1]) + o) = v1;
+                    *reinterpret_cast<f32x4*>(static_cast<float*>(p.out[2]) + o) = v2;
+                }
+        } else {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    const long o = wrow * DH + 32 * ct + 8 * a + 4 * g;
+                    bf16x4 v0, v1, v2;
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        v0[x] = (bf16_t)dk[ct][4 * a + x];
+                        v1[x] = (bf16_t)du[ct][4 * a + x];
+                        v2[x] = (bf16_t)dv[ct][4 * a + x];
+                    }
+                    *reinterpret_cast<bf16x4*>(static_cast<bf16_t*>(p.out[0]) + o) = v0;
+                    *reinterpret_cast<bf16x4*>(static_cast<bf16_t*>(p.out[1]) + o) = v1;
+                    *reinterpret_cast<bf16x4*>(static_cast<bf16_t*>(p.out[2]) + o) = v2;
+                }
+        }
     }
 }
 
@@ -573,31 +607,37 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
 // ------------------------------------------------------------------------------------------------ host side
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-// Token slices of the dK/dU/dV kernel for a workspace of `ws_bytes`: 0 if not even one slice of partials fits.
+// Token slices of the dK/dU/dV kernel for a workspace of `ws_bytes`.  One workgroup fits a CU at a time, so a launch
+// runs in rounds of CUs workgroups; a workgroup costs its share of the token tiles plus a fixed prologue and epilogue
+// (loading its K/U/V blocks, storing 3 x 64 accumulator registers per lane: about 9 tiles' worth).  More slices than
+// one are worth it only where one slice leaves CUs idle; with one slice the kernel writes dK, dU, dV itself and neither
+// partial sums nor the summing pass exist.  Every further slice adds a set of fp32 partial sums that is written and
+// read back once (priced at the time of a token tile per 2.5 MB: about 4 TB/s against 1.25 us per tile).
+constexpr int DW_CUS = 256;             // compute units of an MI355X
+constexpr long DW_FIXED_TILES = 9;      // prologue + epilogue of a workgroup, in token tiles
+constexpr long DW_BYTES_PER_TILE_TIME = 2500000;
 static int pick_nslice(const Dims& d, size_t ws_bytes)
 {
-    // Enough workgroups for ~2 per CU (256 CUs), but at least 8 token tiles per slice.
     const int nblk = d.E * (d.d_e / JB);
     const long cols = (long)((nblk + 3) / 4) * d.Hkuv;
     const long ntile = (long)(d.H / d.Hkuv) * d.B * ((d.S + 31) / 32);
-    long ns = (512 + cols - 1) / cols;
-    if (ns > ntile / 8) ns = ntile / 8;
-    if (ns < 1) ns = 1;
-    if (ns > 64) ns = 64;
     const size_t slice_b = (size_t)3 * d.Hkuv * d.E * d.d_e * d.d_h * sizeof(float);
-    while (ns > 0 && align256((size_t)ns * slice_b) > ws_bytes) --ns;
-    return (int)ns;
+    long best = 1, best_cost = -1;
+    for (long ns = 1; ns <= 64 && (ns == 1 || ns <= ntile / 8); ++ns) {
+        if (ns > 1 && align256((size_t)ns * slice_b) > ws_bytes) break;
+        const long rounds = (cols * ns + DW_CUS - 1) / DW_CUS;
+        const long cost = rounds * ((ntile + ns - 1) / ns + DW_FIXED_TILES) +
+                          (ns > 1 ? ns * (long)(slice_b / DW_BYTES_PER_TILE_TIME) : 0);
+        if (best_cost < 0 || cost < best_cost) { best = ns; best_cost = cost; }
+    }
+    return (int)best;
 }
 
 size_t bwd_workspace_bytes_bf16(const Dims& d)
 {
     const size_t wsz = (size_t)d.Hkuv * d.E * d.d_e * d.d_h;
-    return align256((size_t)pick_nslice(d, ~(size_t)0) * 3 * wsz * sizeof(float));
-}
-
-size_t bwd_min_workspace_bytes_bf16(const Dims& d)
-{
-    return align256((size_t)3 * d.Hkuv * d.E * d.d_e * d.d_h * sizeof(float));
+    const int ns = pick_nslice(d, ~(size_t)0);
+    return ns > 1 ? align256((size_t)ns * 3 * wsz * sizeof(float)) : 0;
 }
 
 template <int DH>
@@ -624,10 +664,9 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
         if (err != hipSuccess) return err;
     }
     const int nslice = pick_nslice(d, ws_bytes);
-    if (nslice < 1) return hipErrorInvalidValue;
     if (phases & PH_BWD_DKDUDV) {
         DwArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R, part,
-                 d.B, d.H, G, d.S, d.E, nbe, nslice, d.tokmaj};
+                 {dK, dU, dV}, grad_w_f32, d.B, d.H, G, d.S, d.E, nbe, nslice, d.tokmaj};
         const int smem = DW_NST * DW_STAGE_B + 128;
         static LdsOptIn optin_full, optin_tail;
         err = d.S % 32 == 0 ? ensure_dynamic_lds(optin_full, (const void*)mhffn_bwd_dkdudv_kernel<DH, false>, smem)
@@ -642,7 +681,7 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }
-    if (phases & PH_BWD_REDUCE) {
+    if ((phases & PH_BWD_REDUCE) && nslice > 1) {
         const long wsz = (long)d.Hkuv * d.E * d.d_e * d.d_h;
         const unsigned rblocks = (unsigned)((wsz / 4 + 255) / 256);
         if (grad_w_f32)

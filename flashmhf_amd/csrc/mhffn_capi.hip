@@ -175,9 +175,9 @@ int mhffn_bwd_static(const void* Q, const void* K, const void* U, const void* V,
     for (const void* p : ptrs)
         if (!aligned16(p)) return MHFFN_ERR_ALIGNMENT;
     const mhffn::Dims d = to_dims(dims, token_layout);
-    // The float32 kernels take exactly the workspace they ask for; the bfloat16 launch uses fewer token slices when the
-    // array holds fewer partial sets than it would like, and needs room for one.
-    const size_t need = dtype == MHFFN_DTYPE_F32 ? mhffn::bwd_workspace_bytes_f32(d) : mhffn::bwd_min_workspace_bytes_bf16(d);
+    // The float32 kernels take exactly the workspace they ask for.  The bfloat16 launch runs with as many token slices
+    // as the array holds partial sums for (with one slice it needs none), so it never exceeds the array.
+    const size_t need = dtype == MHFFN_DTYPE_F32 ? mhffn::bwd_workspace_bytes_f32(d) : 0;
     if (need > MHFFN_STATIC_SCRATCH_BYTES) return MHFFN_ERR_STATIC_SCRATCH;
     void* ws = nullptr;
     if (static_scratch_of_current_device(&ws) != hipSuccess) return MHFFN_ERR_LAUNCH;

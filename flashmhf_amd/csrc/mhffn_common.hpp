@@ -276,8 +276,8 @@ __host__ __device__ inline TokRows tok_rows(int tokmaj, int b, int h, int H, int
 }
 
 size_t fwd_workspace_bytes_bf16(const Dims& d);
-size_t bwd_workspace_bytes_bf16(const Dims& d);       // what the launch uses when it may choose freely
-size_t bwd_min_workspace_bytes_bf16(const Dims& d);   // one token slice of partials: the least launch_bwd_bf16 accepts
+size_t bwd_workspace_bytes_bf16(const Dims& d);       // what the launch uses when it may choose freely (0: one token
+                                                      // slice, no partial sums); with less it runs fewer slices
 hipError_t launch_fwd_bf16(const void* Q, const void* K, const void* U, const void* V, const float* R, void* O,
                            void* ws, const Dims& d, hipStream_t st, int phases);
 hipError_t launch_bwd_bf16(const void* Q, const void* K, const void* U, const void* V, const float* R, const void* dO,

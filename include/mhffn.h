@@ -138,11 +138,12 @@ int mhffn_bwd_layout(const void* Q, const void* K, const void* U, const void* V,
  * partial sums of dK, dU, dV live in a fixed array of MHFFN_STATIC_SCRATCH_BYTES that is part of the library's device
  * code (each GPU the library runs on holds one copy until the process ends).  The call allocates nothing and frees
  * nothing; its first call on a device looks the array's address up once.
- *   - bfloat16: the dK/dU/dV kernel runs with as many token slices as fit the array (fewer than mhffn_bwd would use on
- *     large problems: dK, dU, dV then differ from mhffn_bwd's in the last float32 bits of the partial sums' order, and
- *     the kernel is slower), and needs room for one slice: 3 * Hkuv * E * d_e * d_h * 4 bytes.  Larger problems, and
- *     float32 problems whose mhffn_bwd_workspace_bytes() exceed the array, return MHFFN_ERR_STATIC_SCRATCH before any
- *     launch.
+ *   - bfloat16: the dK/dU/dV kernel runs with as many token slices as the array holds partial sums for (fewer than
+ *     mhffn_bwd would use on some problems: dK, dU, dV then differ from mhffn_bwd's in the last float32 bits of the
+ *     partial sums' order, and the kernel fills the GPU less well); with a single slice it needs no partial sums, so
+ *     no bfloat16 problem is refused.
+ *   - float32 (the correctness instantiation): problems whose mhffn_bwd_workspace_bytes() exceed the array return
+ *     MHFFN_ERR_STATIC_SCRATCH before any launch.
  *   - all calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two threads) race.
  *     Nothing in it has to start at zero (every element read was written by the same call), so it is never cleared. */
 #define MHFFN_STATIC_SCRATCH_BYTES (96u << 20)

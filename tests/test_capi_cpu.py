@@ -61,8 +61,23 @@ def test_check_dims_codes(L, dims, dtype, code):
     assert L.mhffn_check_dims(d, dtype) == code
     if code != 0:
         assert L.mhffn_fwd_workspace_bytes(d, dtype) == 0 and L.mhffn_bwd_workspace_bytes(d, dtype) == 0
+    elif dtype == _capi.DTYPE_F32:
+        assert L.mhffn_bwd_workspace_bytes(d, dtype) > 0     # float32 kernels: partial sums of dK/dU/dV
     else:
-        assert L.mhffn_bwd_workspace_bytes(d, dtype) > 0     # token-slice partials of dK/dU/dV
+        # 11 * 11 * 8 = 968 weight-block columns fill the chip without slicing the tokens: no partial sums
+        assert L.mhffn_bwd_workspace_bytes(d, dtype) == 0
+
+
+def test_backward_workspace_follows_the_token_slice_policy(L):
+    """bfloat16 dK/dU/dV: the tokens are cut into slices only where the weight-block columns alone leave compute units
+    idle; each slice beyond the first costs one float32 copy of dK, dU, dV in the workspace (256-byte aligned)."""
+    one = 3 * 4 * 128                                        # bytes per weight row over dK, dU, dV
+    for dims, slices in (((8, 8, 8, 2048, 128, 11, 352), 1), ((4, 16, 16, 8192, 128, 22, 352), 1),
+                         ((8, 6, 6, 2048, 128, 11, 352), 4), ((2, 4, 4, 1024, 128, 8, 256), 4)):
+        d = _capi.Dims(*dims)
+        rows = dims[2] * dims[5] * dims[6]
+        want = 0 if slices == 1 else -(-slices * rows * one // 256) * 256
+        assert L.mhffn_bwd_workspace_bytes(d, _capi.DTYPE_BF16) == want, (dims, slices)
 
 
 def test_entry_points_validate_before_touching_the_gpu(L):
@@ -73,7 +88,9 @@ def test_entry_points_validate_before_touching_the_gpu(L):
     odd = ctypes.c_void_p(0x1008)
     ok = ctypes.c_void_p(0x1000)
     assert L.mhffn_fwd(odd, ok, ok, ok, ok, ok, ok, 1 << 30, d, 0, null) == _capi.ERR_ALIGNMENT
-    assert L.mhffn_bwd(*([ok] * 11), 0, ok, 16, d, 0, null) == _capi.ERR_WORKSPACE
+    sliced = _capi.Dims(2, 4, 4, 1024, 128, 8, 256)          # a shape whose backward keeps partial sums (4 token slices)
+    assert L.mhffn_bwd(*([ok] * 11), 0, ok, 16, sliced, 0, null) == _capi.ERR_WORKSPACE
+    assert L.mhffn_bwd(*([ok] * 11), 0, null, 1 << 30, sliced, 0, null) == _capi.ERR_WORKSPACE
     assert L.mhffn_bwd(*([ok] * 11), 5, ok, 1 << 30, d, 0, null) == _capi.ERR_DTYPE
     bad = _capi.Dims(1, 2, 2, 64, 128, 2, 65)
     assert L.mhffn_fwd(ok, ok, ok, ok, ok, ok, ok, 1 << 30, bad, 0, null) == _capi.ERR_EXPERT_DIM
@@ -81,7 +98,7 @@ def test_entry_points_validate_before_touching_the_gpu(L):
     assert L.mhffn_fwd_layout(null, null, null, null, null, null, null, 0, d, 0, _capi.TOKENS_BSHD, null, 3) == _capi.ERR_NULL_POINTER
     assert L.mhffn_fwd_layout(ok, ok, ok, ok, ok, ok, ok, 1 << 30, d, 0, 7, null, 3) == _capi.ERR_SHAPE
     assert L.mhffn_bwd_layout(*([ok] * 11), 0, ok, 1 << 30, d, 0, -1, null, 15) == _capi.ERR_SHAPE
-    assert L.mhffn_bwd_layout(*([ok] * 11), 0, ok, 16, d, 0, _capi.TOKENS_BSHD, null, 15) == _capi.ERR_WORKSPACE
+    assert L.mhffn_bwd_layout(*([ok] * 11), 0, ok, 16, sliced, 0, _capi.TOKENS_BSHD, null, 15) == _capi.ERR_WORKSPACE
     # more than 2^31 token rows are rejected (row indices are 32-bit inside the kernels)
     huge = _capi.Dims(4096, 64, 64, 1 << 14, 128, 2, 64)
     assert L.mhffn_check_dims(huge, 0) == _capi.ERR_SHAPE

@@ -1,9 +1,9 @@
 """mhffn_bwd_static (the backward that allocates nothing: its dK/dU/dV partial sums live in a fixed device array inside the
 library) against mhffn_bwd_layout on the same inputs, through the C ABI.  Two calls in a row share the array, the second
 on a smaller problem, so stale partials of the first call would show up in the second.  Where both entry points run the
-same number of token slices every output must be bit-identical; at the full 370M-layer size the fixed array holds fewer
-slices than mhffn_bwd uses, so dK, dU, dV are sums of the same float32 terms in another order (bar: 1e-5 of the
-tensor's largest value; dQ and dR stay bit-identical)."""
+same number of token slices every output must be bit-identical; on a problem for which mhffn_bwd asks for more
+workspace than the fixed array has, the static call runs fewer slices, so dK, dU, dV are sums of the same float32 terms
+in another order (bar: 1e-5 of the tensor's largest value; dQ and dR stay bit-identical)."""
 import ctypes
 
 import pytest
@@ -45,7 +45,7 @@ def _run_both(shape, seed, dtype, wdtype, layout=0):
 
 def test_static_scratch_backward_matches_the_workspace_backward_on_two_calls_in_a_row():
     from flashmhf_amd import _capi
-    # first a problem whose partial sums fill the array to the last byte (8 slices of 12 MiB), then a smaller one, then float32
+    # first a problem whose partial sums fill half the array (4 slices of 12 MiB), then smaller ones, then float32
     calls = [((2, 4, 1024, 128, 8, 256, 4), 41, torch.bfloat16, torch.bfloat16, _capi.TOKENS_BHSD),
              ((1, 4, 300, 128, 2, 64, 2), 42, torch.bfloat16, torch.float32, _capi.TOKENS_BSHD),
              ((2, 3, 70, 96, 3, 96, 3), 43, torch.bfloat16, torch.bfloat16, _capi.TOKENS_BHSD),
@@ -59,9 +59,10 @@ def test_static_scratch_backward_matches_the_workspace_backward_on_two_calls_in_
             assert torch.equal(a, b), name
 
 
-def test_static_scratch_backward_at_the_full_370m_layer_size_with_fewer_token_slices():
+def test_static_scratch_backward_with_fewer_token_slices_than_the_workspace_backward():
     from flashmhf_amd import _capi
-    ref, got, ws_bytes = _run_both((8, 8, 2048, 128, 11, 352, 8), 45, torch.bfloat16, torch.float32)
+    # 6 heads of the 370M layer: mhffn_bwd asks for 4 slices of 34 MiB, the fixed 96 MiB array holds 2
+    ref, got, ws_bytes = _run_both((8, 6, 2048, 128, 11, 352, 6), 45, torch.bfloat16, torch.float32)
     assert ws_bytes > _capi.STATIC_SCRATCH_BYTES, "this case is meant to need fewer token slices than mhffn_bwd uses"
     assert torch.equal(got[0], ref[0]) and torch.equal(got[4], ref[4])
     for name, a, b in zip(("dK", "dU", "dV"), got[1:4], ref[1:4]):
@@ -76,9 +77,10 @@ def test_static_scratch_backward_at_the_full_370m_layer_size_with_fewer_token_sl
 def test_static_scratch_backward_rejects_what_does_not_fit_before_any_launch():
     from flashmhf_amd import _capi
     L = _capi.lib()
-    dims = _capi.Dims(1, 16, 16, 64, 128, 22, 352)       # one slice of partials: 3 * 16*22*352*128 * 4 B = 190 MB
+    dims = _capi.Dims(1, 16, 16, 64, 128, 22, 352)       # float32 partial sums: 3 * 16*22*352*128 * 4 B = 190 MB
     buf = torch.zeros(1024, device=DEV)
     p = buf.data_ptr()
-    rc = L.mhffn_bwd_static(p, p, p, p, p, p, p, p, p, p, p, 0, dims, 0, 0, None)
+    rc = L.mhffn_bwd_static(p, p, p, p, p, p, p, p, p, p, p, _capi.DTYPE_F32, dims, _capi.DTYPE_F32, 0, None)
     assert rc == _capi.ERR_STATIC_SCRATCH
     assert "mhffn_bwd_static" in _capi.strerror(rc)
+    assert L.mhffn_bwd_workspace_bytes(dims, _capi.DTYPE_F32) > _capi.STATIC_SCRATCH_BYTES
