@@ -199,6 +199,7 @@ HARDWARE = {"fwd_main": 3, "bwd_dqdr": 5, "bwd_dkdudv": 6}
 # traffic null: the record no longer describes the kernels being timed.
 TRAFFIC_KERNELS = {"fwd_main": "mhffn_fwd_kernel", "bwd_dqdr": "mhffn_bwd_dqdr_kernel",
                    "bwd_dkdudv": "mhffn_bwd_dkdudv_kernel", "bwd_reduce": "reduce_partials_kernel"}
+TRAFFIC_SOURCES = ("mhffn_bwd.hip", "mhffn_common.hpp", "mhffn_fwd.hip")
 COPY_KERNEL, COPY_BYTES = "__amd_rocclr_copyBuffer", 256 << 20
 
 
@@ -210,10 +211,9 @@ def kernel_source_hash():
     import hashlib
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, "flashmhf_amd", "csrc")
-    for name in sorted(os.listdir(csrc)):
-        if name.endswith((".hip", ".hpp")):
-            h.update(name.encode())
-            h.update(open(os.path.join(csrc, name), "rb").read())
+    for name in TRAFFIC_SOURCES:                     # the files the four measured kernels are compiled from
+        h.update(name.encode())
+        h.update(open(os.path.join(csrc, name), "rb").read())
     return h.hexdigest()
 
 
