@@ -254,7 +254,7 @@ def write_traffic_record(workload, fetch_csv, write_csv, out_path):
     w_scale = (COPY_BYTES / 1024.0) / copy_reading(write_csv, "WRITE_SIZE")
     rec = {"workload": workload, "kernel_source_sha256": kernel_source_hash(),
            "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv -d <dir> -o p -- python3 bench.py "
-                      f"--workload {workload} --no-cpu --steps 2 --warmup 1 --calibrate-copy ; python3 bench.py --workload "
+                      f"--workload {workload} --no-cpu --no-others --steps 2 --warmup 1 --calibrate-copy ; python3 bench.py --workload "
                       f"{workload} --traffic-from <fetch csv> <write csv>",
            "scale": {"FETCH_SIZE": f_scale, "WRITE_SIZE": w_scale,
                      "reference": "256 MiB device copy (__amd_rocclr_copyBuffer) reads and writes 262144 KiB per launch"},
@@ -416,7 +416,9 @@ def bench_model(w, args, dev):
         "fused_ffn_credited_tflops_if_it_were_the_whole_step": ffn_flops / (ms * 1e-3) / 1e12,
         "roofline": None, "cpu_baseline": None,
     }
-    print(json.dumps(out))
+    del model
+    torch.cuda.empty_cache()
+    return out
 
 
 def bench_prologue(w, args, dev):
@@ -493,7 +495,7 @@ def bench_prologue(w, args, dev):
         out["cpu_baseline"] = {"value": sum(alg.values()) * frac / med / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
                                "kind": "port", "sample": f"oracle head_norm_gate + autograd, fp32, B1xS1024 tokens of the "
                                                          f"same heads, median of 5 runs, {med * 1e3:.1f} ms"}
-    print(json.dumps(out))
+    return out
 
 
 def main():
@@ -504,6 +506,9 @@ def main():
                     help="untimed steps first: the GPU clock needs some tens of milliseconds of load to settle")
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-others", action="store_true",
+                    help="default workload only: skip the short runs of the other configurations (c1, c3, head prologue, "
+                         "c4 decoder) that are appended to the JSON line as `other_workloads`")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy a few times (known-size reference for HBM traffic counters)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
@@ -529,7 +534,25 @@ def main():
             dst.copy_(src)           # reads 256 MiB, writes 256 MiB per launch
         torch.cuda.synchronize()
         del src, dst
-    w = WORKLOADS[args.workload]
+    out = run_workload(args.workload, args, dev)
+    if args.workload == "c2" and not args.no_others:
+        # the other configurations, short runs without the CPU legs, so that one default invocation records them all
+        sub = argparse.Namespace(**{**vars(args), "no_cpu": True, "steps": 20, "warmup": 5})
+        keep = ("value", "unit", "ms_per_step", "steps", "warmup", "config", "frac_of_mfma_peak", "tokens_per_s", "peak_hbm_bytes",
+                "peak_memory_bytes", "swiglu_2048_5504_peak_hbm_bytes_beyond_inputs", "kernels", "roofline", "loss")
+        out["other_workloads"] = {}
+        for name in ("c1", "c3", "c2_prologue", "c3_prologue", "c4"):
+            sub.workload = name
+            sub.steps, sub.warmup = (5, 2) if name == "c4" else (20, 5)
+            r = run_workload(name, sub, dev, light=True)
+            out["other_workloads"][name] = {k: r[k] for k in keep if k in r}
+    print(json.dumps(out))
+
+
+def run_workload(name, args, dev, light=False):
+    """One workload -> its result record.  light: no clock/power sampling, no matrix-loop probe, no autograd-operator timing."""
+    from flashmhf_amd import mhffn_backward, mhffn_forward
+    w = WORKLOADS[name]
     if w["passes"] == "model":
         return bench_model(w, args, dev)
     if w["passes"] == "prologue":
@@ -569,7 +592,7 @@ def main():
     torch.cuda.synchronize()
     per_step = sorted(a.elapsed_time(b) for a, b in evs)
     timing = {"median_ms": per_step[len(per_step) // 2], "min_ms": per_step[0]}
-    if bwd:
+    if bwd and not light:
         from flashmhf_amd import FlashMLPMoE
         op = FlashMLPMoE()
         leaves = [t.detach().clone().requires_grad_(True) for t in (Q, K, U, V, R)]
@@ -581,11 +604,11 @@ def main():
 
         timing["autograd_op_ms"] = time_events(autograd_step, min(args.steps, 100))
 
-    kt, kstate = kernel_timings(w, ins)
-    mfma_loop, probe_state = measured_mfma_peak_tflops(dev)
+    kt, kstate = kernel_timings(w, ins, sample_state=not light)
+    mfma_loop, probe_state = (None, None) if light else measured_mfma_peak_tflops(dev)
     dom = max(CREDIT, key=lambda k: kt.get(k, 0.0))
     ach = CREDIT[dom] * f1(w) / (kt[dom] * 1e-3) / 1e12
-    traffic, traffic_note = recorded_traffic(args.workload, dom)
+    traffic, traffic_note = recorded_traffic(name, dom)
     roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": ach / PEAK_BF16_TFLOPS, "traffic": traffic, "traffic_source": traffic_note,
                 "hardware_tflops": HARDWARE[dom] * f1(w) / (kt[dom] * 1e-3) / 1e12}
@@ -595,18 +618,18 @@ def main():
                for k, v in kt.items()}
 
     out = {
-        "metric": "fused MH-FFN fwd+bwd TFLOP/s (% MFMA peak) + peak HBM, 370M layer, 1 GPU" if args.workload == "c2"
-                  else f"fused MH-FFN {w['passes']} TFLOP/s, workload {args.workload}",
+        "metric": "fused MH-FFN fwd+bwd TFLOP/s (% MFMA peak) + peak HBM, 370M layer, 1 GPU" if name == "c2"
+                  else f"fused MH-FFN {w['passes']} TFLOP/s, workload {name}",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {w['label']}", "credited_flops_per_step": flops,
+        "config": {"workload": f"{name}: {w['label']}", "credited_flops_per_step": flops,
                    "flop_convention": "11*F1 fwd+bwd (3 fwd + 8 bwd), F1=2*T*H*E*d_e*d_h"},
         "frac_of_mfma_peak": tflops / PEAK_BF16_TFLOPS,
         "measured_mfma_loop_tflops": mfma_loop,
         "measured_mfma_loop_under_load": probe_state,
         "nominal_peak_clock_mhz": 2400,
-        "frac_of_measured_mfma_loop": tflops / mfma_loop,
+        "frac_of_measured_mfma_loop": tflops / mfma_loop if mfma_loop else None,
         "tokens_per_s": tokens / (ms * 1e-3),
         "peak_hbm_bytes": {"beyond_inputs": int(peak_extra), "inputs": int(base_mem),
                            "forbidden_intermediate_bytes_one_tensor": tokens * w["H"] * w["E"] * w["d_e"] * 2},
@@ -614,12 +637,14 @@ def main():
         "kernels": kernels,
         "timing": timing,
     }
-    if args.workload == "c3":
+    if name == "c3":
         out["swiglu_2048_5504_peak_hbm_bytes_beyond_inputs"] = swiglu_peak_bytes(tokens, 2048, 5504, dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(w)
         out["cpu_baseline_c0"] = cpu_baseline_c0()
-    print(json.dumps(out))
+    del ins, Q, K, U, V, R, dO
+    torch.cuda.empty_cache()
+    return out
 
 
 if __name__ == "__main__":
