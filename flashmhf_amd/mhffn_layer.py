@@ -101,6 +101,14 @@ class MHFFNLayer(nn.Module):
             w = src.view(self.num_experts * self.expert_dim, self.num_kuv_heads, self.head_dim).transpose(0, 1)
             dst.copy_(w.reshape(self.num_kuv_heads, self.num_experts, self.expert_dim, self.head_dim))
 
+    @torch.no_grad()
+    def export_reference_weights(self):
+        """The inverse of load_reference_weights: (gate_weight, up_weight, down_weight), each [E*d_e, Hkuv*d_h] as the
+        reference stores them (modeling_mhffnmoe.py:343-345), so a model trained here can be saved in its format."""
+        rows = self.num_experts * self.expert_dim
+        return tuple(w.detach().reshape(self.num_kuv_heads, rows, self.head_dim).transpose(0, 1)
+                     .reshape(rows, self.num_kuv_heads * self.head_dim).clone() for w in (self.K, self.U, self.V))
+
     def heads_and_gate(self, x):
         """Q as the [B, H, S, d_h] view of the projection's [B, S, H, d_h] memory, and R [B, H, S, E] fp32."""
         B, S, _ = x.shape

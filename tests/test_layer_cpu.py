@@ -61,6 +61,15 @@ def test_load_reference_weights_puts_each_head_and_expert_where_the_kernels_expe
             assert torch.equal(layer.V[hk, e], down[e * de:(e + 1) * de, hk * dh:(hk + 1) * dh])
 
 
+def test_export_reference_weights_inverts_the_load():
+    H, Hk, dh, E, de = 4, 2, 8, 3, 5
+    layer = MHFFNLayer(H * dh, H, E, de, Hk, op=_eager_op)
+    gate, up, down = (torch.randn(E * de, Hk * dh) for _ in range(3))
+    layer.load_reference_weights(gate, up, down)
+    for got, want in zip(layer.export_reference_weights(), (gate, up, down)):
+        assert got.shape == want.shape and got.is_contiguous() and torch.equal(got, want)
+
+
 def test_rmsnorm_and_gate_closed_forms():
     x = torch.tensor([[3.0, 4.0]])
     assert torch.allclose(RMSNorm((2,), eps=0.0)(x), x / (12.5 ** 0.5))
