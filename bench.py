@@ -117,16 +117,45 @@ def kernel_timings(w, ins, n=50, sample_state=True):
     return out, state
 
 
+def device_sysfs_dir():
+    """sysfs directory of the GPU torch runs on (cuda:0), found through its PCI address; with that unknown, the only
+    card of the machine; None when several cards are visible and none can be matched."""
+    import glob
+    try:
+        pr = torch.cuda.get_device_properties(0)
+        d = f"/sys/bus/pci/devices/{pr.pci_domain_id:04x}:{pr.pci_bus_id:02x}:{pr.pci_device_id:02x}.0"
+        if os.path.exists(os.path.join(d, "pp_dpm_sclk")):
+            return d
+    except (AttributeError, RuntimeError):
+        pass
+    cards = sorted(os.path.dirname(f) for f in glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+    return cards[0] if len(cards) == 1 else None
+
+
+def settle_clock(fn, ms):
+    """Runs `fn` back to back for at least `ms` milliseconds (untimed) and returns the time spent: the shader clock and
+    the power controller need some tens of milliseconds of the workload itself before they stop moving."""
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3
+
+
 def device_state_under(fn, seconds=0.5):
     """Shader clock (MHz) and package power (W) as the driver reports them (sysfs pp_dpm_sclk, hwmon power1_input)
     while `fn` is launched back to back for `seconds`: median of the samples taken after the first 100 ms.  The clock a
     kernel is given depends on the kernel: under matrix-heavy load the package sits at its power limit and the clock
     settles well below the 2.4 GHz the nominal peak is quoted at.  Returns None where the files cannot be read."""
-    import glob
     import threading
-    sclk = glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")
-    pwr = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")
-    cap = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap")
+    card = device_sysfs_dir()
+    if card is None:
+        return None
+    import glob
+    sclk = glob.glob(os.path.join(card, "pp_dpm_sclk"))
+    pwr = glob.glob(os.path.join(card, "hwmon", "hwmon*", "power1_input"))
+    cap = glob.glob(os.path.join(card, "hwmon", "hwmon*", "power1_cap"))
     if not sclk:
         return None
     samples, stop = [], threading.Event()
@@ -451,6 +480,7 @@ def bench_prologue(w, args, dev):
         fwd()
         bwd()
 
+    pre_warm_ms = settle_clock(step, args.pre_warm_ms)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -468,6 +498,7 @@ def bench_prologue(w, args, dev):
         "metric": "MH-FFN head prologue fwd+bwd GB/s (algorithmic bytes), 1 GPU", "value": sum(alg.values()) / (ms * 1e-3) / 1e9,
         "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "pre_warm_ms": pre_warm_ms,
         "config": {"workload": f"{args.workload}: {w['label']}", "algorithmic_bytes_per_step": sum(alg.values())},
         "tokens_per_s": B * S / (ms * 1e-3),
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -504,6 +535,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50,
                     help="untimed steps first: the GPU clock needs some tens of milliseconds of load to settle")
+    ap.add_argument("--pre-warm-ms", type=float, default=200.0,
+                    help="before the counted warm-up steps, run the workload untimed for this long so that the timed steps "
+                         "do not fall into the clock's start-up transient (reported as pre_warm_ms)")
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true",
@@ -538,7 +572,7 @@ def main():
     if args.workload == "c2" and not args.no_others:
         # the other configurations, short runs without the CPU legs, so that one default invocation records them all
         sub = argparse.Namespace(**{**vars(args), "no_cpu": True, "steps": 20, "warmup": 5})
-        keep = ("value", "unit", "ms_per_step", "steps", "warmup", "config", "frac_of_mfma_peak", "tokens_per_s", "peak_hbm_bytes",
+        keep = ("value", "unit", "ms_per_step", "steps", "warmup", "pre_warm_ms", "config", "frac_of_mfma_peak", "tokens_per_s", "peak_hbm_bytes",
                 "peak_memory_bytes", "swiglu_2048_5504_peak_hbm_bytes_beyond_inputs", "kernels", "roofline", "loss")
         out["other_workloads"] = {}
         for name in ("c1", "c3", "c2_prologue", "c3_prologue", "c4"):
@@ -567,6 +601,7 @@ def run_workload(name, args, dev, light=False):
             return O, mhffn_backward(Q, K, U, V, R, dO, grad_w_dtype=torch.bfloat16)
         return O
 
+    pre_warm_ms = settle_clock(step, args.pre_warm_ms)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -622,7 +657,7 @@ def run_workload(name, args, dev, light=False):
                   else f"fused MH-FFN {w['passes']} TFLOP/s, workload {name}",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "bf16", "data": "synthetic", "pre_warm_ms": pre_warm_ms,
         "config": {"workload": f"{name}: {w['label']}", "credited_flops_per_step": flops,
                    "flop_convention": "11*F1 fwd+bwd (3 fwd + 8 bwd), F1=2*T*H*E*d_e*d_h"},
         "frac_of_mfma_peak": tflops / PEAK_BF16_TFLOPS,

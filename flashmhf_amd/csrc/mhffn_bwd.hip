@@ -223,11 +223,10 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     const int nblk = p.E * p.nbe;
     const int jblk = blockIdx.y * 4 + wave;
     const bool active = jblk < nblk;
-    const int jb_c = active ? jblk : nblk - 1;        // idle waves of the last column recompute the last block
+    const int jb_c = active ? jblk : nblk - 1;        // waves of the last column without a block: addresses stay valid
     const int e_w = jb_c / p.nbe;
     const long wrow = ((long)hk * nblk + jb_c) * JB + l32;      // this lane's row of K/U/V (column j of the products)
 
-    // The K, U and V blocks stay in registers as MFMA B operands for the whole kernel (K, U in accumulation registers).
     float* sZero = reinterpret_cast<float*>(smem_raw + DW_NST * DW_STAGE_B);   // 32 zero gate values
     if (tid < 32) sZero[tid] = 0.0f;
     // The first step contracts a tile that does not exist (zero gate values) out of the last stage, which no load has
@@ -238,21 +237,9 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         u32x4* last_stage = reinterpret_cast<u32x4*>(smem_raw + (DW_NST - 1) * DW_STAGE_B);
         for (int i = tid; i < 2 * TILE_B / 16; i += 256) last_stage[i] = z;
     }
-    bf16x8 kB[KS], uB[KS];
-    bf16x8 vR[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        kB[ks] = *reinterpret_cast<const bf16x8*>(p.K + wrow * DH + ks * 16 + 8 * g);
-        uB[ks] = *reinterpret_cast<const bf16x8*>(p.U + wrow * DH + ks * 16 + 8 * g);
-        vR[ks] = *reinterpret_cast<const bf16x8*>(p.V + wrow * DH + ks * 16 + 8 * g);
-    }
-
-    f32x16 dk[CT], du[CT], dv[CT];
-#pragma unroll
-    for (int i = 0; i < CT; ++i)
-#pragma unroll
-        for (int x = 0; x < 16; ++x) { dk[i][x] = 0.0f; du[i][x] = 0.0f; dv[i][x] = 0.0f; }
-
+    // These clears are ordinary LDS stores that other waves read in step 0, and the barriers of the token loop are bare
+    // (no wait on this wave's own LDS stores): one fenced barrier here publishes them, once per workgroup.
+    __syncthreads();
     const int nS = (p.S + 31) / 32;
     const int ntile = p.G * p.B * nS;
     const int t_begin = (int)((long)ntile * z / p.nslice), t_end = (int)((long)ntile * (z + 1) / p.nslice);
@@ -336,6 +323,51 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         float* sR = reinterpret_cast<float*>(smem_raw + sidx * DW_STAGE_B + 2 * TILE_B);
         if (l32 >= nvalid) sR[wave * 64 + lane] = 0.0f;
     };
+
+    // First two tiles of the slice; the third is fired behind the first barrier of the loop.
+    prepare_tile();
+    int nv0 = fire_tile(0);
+    prepare_tile();
+    int nv1 = fire_tile(1), nv2 = 32, nv3 = 32;        // valid rows of the tile in each stage
+    if constexpr (!TAIL) prepare_tile();
+
+    if (!active) {
+        // A wave of a head's last column that has no block: it keeps up its share of the tile fills and the barriers
+        // (as many as the working waves pass, nt + 1) and issues no matrix instruction.
+        for (int k = 0; k <= nt; ++k) {
+            const int st = k & 3;
+            wait_vmcnt<0>();
+            if constexpr (TAIL) {
+                const int nvalid = st == 0 ? nv0 : (st == 1 ? nv1 : (st == 2 ? nv2 : nv3));
+                if (nvalid < 32) zero_tail(st, nvalid);
+            }
+            __builtin_amdgcn_s_barrier();
+            if constexpr (TAIL) prepare_tile();
+            const int nvn = fire_tile((st + 2) & 3);
+            if constexpr (!TAIL) prepare_tile();
+            if constexpr (TAIL) {
+                if (st == 0) nv2 = nvn; else if (st == 1) nv3 = nvn; else if (st == 2) nv0 = nvn; else nv1 = nvn;
+            }
+        }
+        wait_vmcnt<0>();
+        return;
+    }
+
+    // The K, U and V blocks stay in registers as MFMA B operands for the whole kernel (K, U in accumulation registers).
+    bf16x8 kB[KS], uB[KS];
+    bf16x8 vR[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        kB[ks] = *reinterpret_cast<const bf16x8*>(p.K + wrow * DH + ks * 16 + 8 * g);
+        uB[ks] = *reinterpret_cast<const bf16x8*>(p.U + wrow * DH + ks * 16 + 8 * g);
+        vR[ks] = *reinterpret_cast<const bf16x8*>(p.V + wrow * DH + ks * 16 + 8 * g);
+    }
+
+    f32x16 dk[CT], du[CT], dv[CT];
+#pragma unroll
+    for (int i = 0; i < CT; ++i)
+#pragma unroll
+        for (int x = 0; x < 16; ++x) { dk[i][x] = 0.0f; du[i][x] = 0.0f; dv[i][x] = 0.0f; }
 
     const int fr = swz16(l32);
     const TrLane<CT> trl = make_tr_lane<CT, 4, 8>(lane);
@@ -496,11 +528,6 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     f32x16 mA, nA, dA_, mB, nB, dB_;
 #pragma unroll
     for (int x = 0; x < 16; ++x) { mA[x] = 0.0f; nA[x] = 0.0f; dA_[x] = 0.0f; mB[x] = 0.0f; nB[x] = 0.0f; dB_[x] = 0.0f; }
-    prepare_tile();
-    int nv0 = fire_tile(0);
-    prepare_tile();
-    int nv1 = fire_tile(1), nv2 = 32, nv3 = 32;        // valid rows of the tile in each stage
-    if constexpr (!TAIL) prepare_tile();               // tile 2: fired behind the first barrier
     auto sync_step = [&](auto st_c, int nvalid, int& nv_next) {
         constexpr int ST = decltype(st_c)::value;
         // All of this wave's loads, not only the older tile's: a partial count (the next tile's loads still in flight)
@@ -519,21 +546,35 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
     using I3 = std::integral_constant<int, 3>;
-    // nt + 1 steps are needed (step k contracts tile k-1); the count is padded to a multiple of 4 with phantom steps
-    // whose products are computed on whatever the stage holds and contracted with a zero gate.
-    for (int k = 0; k <= nt; k += 4) {
-        sync_step(I0{}, nv0, nv2);
-        step(I0{}, I3{}, mA, nA, dA_, mB, nB, dB_, k > 0);
-        sync_step(I1{}, nv1, nv3);
-        step(I1{}, I0{}, mB, nB, dB_, mA, nA, dA_, k < nt);
-        sync_step(I2{}, nv2, nv0);
-        step(I2{}, I1{}, mA, nA, dA_, mB, nB, dB_, k + 1 < nt);
-        sync_step(I3{}, nv3, nv1);
-        step(I3{}, I2{}, mB, nB, dB_, mA, nA, dA_, k + 2 < nt);
+    // nt + 1 steps (step k contracts tile k-1), in trips of four (one per LDS stage) and a remainder of up to three.
+    {
+        int k = 0;
+        for (; k + 3 <= nt; k += 4) {
+            sync_step(I0{}, nv0, nv2);
+            step(I0{}, I3{}, mA, nA, dA_, mB, nB, dB_, k > 0);
+            sync_step(I1{}, nv1, nv3);
+            step(I1{}, I0{}, mB, nB, dB_, mA, nA, dA_, true);
+            sync_step(I2{}, nv2, nv0);
+            step(I2{}, I1{}, mA, nA, dA_, mB, nB, dB_, true);
+            sync_step(I3{}, nv3, nv1);
+            step(I3{}, I2{}, mB, nB, dB_, mA, nA, dA_, true);
+        }
+        if (k <= nt) {
+            sync_step(I0{}, nv0, nv2);
+            step(I0{}, I3{}, mA, nA, dA_, mB, nB, dB_, k > 0);
+            if (k + 1 <= nt) {
+                sync_step(I1{}, nv1, nv3);
+                step(I1{}, I0{}, mB, nB, dB_, mA, nA, dA_, true);
+                if (k + 2 <= nt) {
+                    sync_step(I2{}, nv2, nv0);
+                    step(I2{}, I1{}, mA, nA, dA_, mB, nB, dB_, true);
+                }
+            }
+        }
     }
     wait_vmcnt<0>();
 
-    if (active) {
+    {
         // dK^T registers 4a+b of row tile ct: c = 32ct + 8a + 4g + b, column j = l32 -> runs of 4 along c.
         const long wsz = (long)gridDim.x * nblk * JB * DH;   // elements of one weight tensor
         if (p.nslice > 1) {                                  // fp32 partial sums of this token slice

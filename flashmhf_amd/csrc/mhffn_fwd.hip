@@ -229,8 +229,8 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
         mfma_result_fence(mA[0], nA[0], mA[1]);   // the element-wise code of step 0 reads these results
         mfma_result_fence(nA[1]);
     }
-    // Four blocks per trip (one per LDS stage; the two M/N register sets alternate), then one last pair on stages 0, 1
-    // where the count leaves one or two blocks; an odd count ends in a phantom block whose gate value is 0.
+    // Four blocks per trip (one per LDS stage; the two M/N register sets alternate), then the last one to three.  (The
+    // step of the last block still computes first products, of the block its prefetch clamped to; nothing reads them.)
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
     using S2 = std::integral_constant<int, 2>;
@@ -239,7 +239,7 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     auto advance = [&]() {
         if (++jb == p.nbe) { jb = 0; ++e; }
     };
-    for (; blk + 2 < nblk; blk += 4) {
+    for (; blk + 4 <= nblk; blk += 4) {
         step(S0{}, blk, e, mA, nA, mB, nB);
         advance();
         step(S1{}, blk + 1, e, mB, nB, mA, nA);
@@ -252,7 +252,11 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     if (blk < nblk) {
         step(S0{}, blk, e, mA, nA, mB, nB);
         advance();
-        step(S1{}, blk + 1, e, mB, nB, mA, nA);
+        if (blk + 1 < nblk) {
+            step(S1{}, blk + 1, e, mB, nB, mA, nA);
+            advance();
+            if (blk + 2 < nblk) step(S2{}, blk + 2, e, mA, nA, mB, nB);
+        }
     }
     wait_vmcnt<0>();      // drain the phantom prefetches before the workgroup's LDS is released
 

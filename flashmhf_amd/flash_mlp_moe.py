@@ -13,17 +13,30 @@ is before the caller's ``.contiguous()`` (models/flashmhf/modeling_mhffnmoe.py:3
 and O (and dQ) come back in the same token-major layout, so ``O.transpose(1,2).contiguous().view(B,S,hid)`` (:408) copies
 nothing.
 """
+import contextlib
+import functools
+
 import torch
 
 from . import _capi
 
 
-def _dims(Q, K):
+@functools.lru_cache(maxsize=512)
+def _plan(B, H, Hk, S, dh, E, de, code):
+    """(extents struct, forward workspace bytes, backward workspace bytes) of one problem shape, validated once by the
+    library (raises the reference's exception types); later calls with the same shape cost a dictionary lookup."""
+    L = _capi.lib()
+    dims = _capi.Dims(B, H, Hk, S, dh, E, de)
+    _capi.raise_for_code(L.mhffn_check_dims(dims, code), "mhffn")
+    return dims, L.mhffn_fwd_workspace_bytes(dims, code), L.mhffn_bwd_workspace_bytes(dims, code)
+
+
+def _plan_for(Q, K):
     B, H, S, dh = Q.shape
     Hk, E, de, dh2 = K.shape
     if dh2 != dh:
         raise RuntimeError(f"head dim mismatch: Q has {dh}, K has {dh2}")
-    return _capi.Dims(B, H, Hk, S, dh, E, de)
+    return _plan(B, H, Hk, S, dh, E, de, _capi.torch_dtype_code(Q.dtype))
 
 
 def _check_inputs(Q, K, U, V, R):
@@ -65,8 +78,19 @@ def _as_layout(t, layout):
     return t.contiguous()
 
 
+_NO_GUARD = contextlib.nullcontext()
+
+
 def _ws(nbytes, device):
-    return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)
+    """(pointer, size) of a workspace: a null pointer where the launch needs none."""
+    if nbytes == 0:
+        return None, 0
+    return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
+
+
+def _device_guard(device):
+    """The library launches on the current device: switch only when the tensors live on another one."""
+    return _NO_GUARD if device.index == torch.cuda.current_device() else torch.cuda.device(device)
 
 
 def mhffn_forward(Q, K, U, V, R):
@@ -74,17 +98,14 @@ def mhffn_forward(Q, K, U, V, R):
     _check_inputs(Q, K, U, V, R)
     layout, Q = _token_layout(Q)
     K, U, V, R = (t.contiguous() for t in (K, U, V, R))
-    L = _capi.lib()
-    dims = _dims(Q, K)
-    code = _capi.torch_dtype_code(Q.dtype)
-    _capi.raise_for_code(L.mhffn_check_dims(dims, code), "mhffn_fwd")
+    dims, fwd_bytes, _ = _plan_for(Q, K)
     O = torch.empty_strided(Q.shape, Q.stride(), dtype=Q.dtype, device=Q.device)
-    nbytes = L.mhffn_fwd_workspace_bytes(dims, code)
-    ws = _ws(nbytes, Q.device)
-    with torch.cuda.device(Q.device):
-        rc = L.mhffn_fwd_layout(Q.data_ptr(), K.data_ptr(), U.data_ptr(), V.data_ptr(), R.data_ptr(), O.data_ptr(),
-                                ws.data_ptr(), ws.numel(), dims, code, layout,
-                                torch.cuda.current_stream().cuda_stream, _capi.FWD_ALL)
+    ws, ws_bytes = _ws(fwd_bytes, Q.device)
+    with _device_guard(Q.device):
+        rc = _capi.lib().mhffn_fwd_layout(Q.data_ptr(), K.data_ptr(), U.data_ptr(), V.data_ptr(), R.data_ptr(),
+                                          O.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes, dims,
+                                          _capi.torch_dtype_code(Q.dtype), layout,
+                                          torch.cuda.current_stream().cuda_stream, _capi.FWD_ALL)
     _capi.raise_for_code(rc, "mhffn_fwd")
     return O
 
@@ -97,19 +118,18 @@ def mhffn_backward(Q, K, U, V, R, dO, grad_w_dtype=torch.bfloat16):
     layout, Q = _token_layout(Q)
     K, U, V, R = (t.contiguous() for t in (K, U, V, R))
     dO = _as_layout(dO.to(Q.dtype), layout)
-    L = _capi.lib()
-    dims = _dims(Q, K)
-    code = _capi.torch_dtype_code(Q.dtype)
-    _capi.raise_for_code(L.mhffn_check_dims(dims, code), "mhffn_bwd")
+    dims, _, bwd_bytes = _plan_for(Q, K)
     dQ = torch.empty_strided(Q.shape, Q.stride(), dtype=Q.dtype, device=Q.device)
     dK, dU, dV = (torch.empty(K.shape, dtype=grad_w_dtype, device=K.device) for _ in range(3))
     dR = torch.empty_like(R)
-    ws = _ws(L.mhffn_bwd_workspace_bytes(dims, code), Q.device)
-    with torch.cuda.device(Q.device):
-        rc = L.mhffn_bwd_layout(Q.data_ptr(), K.data_ptr(), U.data_ptr(), V.data_ptr(), R.data_ptr(), dO.data_ptr(),
-                                dQ.data_ptr(), dK.data_ptr(), dU.data_ptr(), dV.data_ptr(), dR.data_ptr(),
-                                _capi.torch_dtype_code(grad_w_dtype), ws.data_ptr(), ws.numel(), dims, code, layout,
-                                torch.cuda.current_stream().cuda_stream, _capi.BWD_ALL)
+    ws, ws_bytes = _ws(bwd_bytes, Q.device)
+    with _device_guard(Q.device):
+        rc = _capi.lib().mhffn_bwd_layout(Q.data_ptr(), K.data_ptr(), U.data_ptr(), V.data_ptr(), R.data_ptr(),
+                                          dO.data_ptr(), dQ.data_ptr(), dK.data_ptr(), dU.data_ptr(), dV.data_ptr(),
+                                          dR.data_ptr(), _capi.torch_dtype_code(grad_w_dtype),
+                                          ws.data_ptr() if ws is not None else None, ws_bytes, dims,
+                                          _capi.torch_dtype_code(Q.dtype), layout,
+                                          torch.cuda.current_stream().cuda_stream, _capi.BWD_ALL)
     _capi.raise_for_code(rc, "mhffn_bwd")
     return dQ, dK, dU, dV, dR
 
