@@ -39,9 +39,10 @@ def build_lib(verbose=False, jobs=4):
         if verbose:
             print(" ".join(cmd), flush=True)
         r = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
-        other = [ln for ln in r.stderr.splitlines()
-                 if "packed-fp32-ops" not in ln and "kernel-resource-usage" not in ln and (r.returncode or "warning" in ln or "error" in ln)]
-        if other:
+        # everything the compiler said except the resource-usage remarks and the host pass's note on the packed-fp32
+        # feature: a warning keeps its source line and caret
+        other = [ln for ln in r.stderr.splitlines() if "packed-fp32-ops" not in ln and "-Rpass-analysis" not in ln]
+        if other and (r.returncode or any("warning" in ln or "error" in ln for ln in other)):
             print("\n".join(other), file=sys.stderr, flush=True)
         if r.returncode:
             raise subprocess.CalledProcessError(r.returncode, cmd)
@@ -77,12 +78,29 @@ def parse_resource_usage(stderr_text):
     return usage
 
 
+# Kernels whose code assumes that every value stays in registers, as (name fragment, instantiations expected).
+EXPECTED_KERNELS = (
+    ("mhffn_fwd_kernel", 3), ("mhffn_bwd_dqdr_kernel", 3), ("mhffn_bwd_dkdudv_kernel", 6),
+    ("mhffn_gate_fwd_kernel", 12), ("mhffn_gate_bwd_kernel", 12),
+)
+# The one instantiation known to spill: head prologue backward for d_h = 128 with more than 32 experts and RMSNorm
+# (<128, 2, true>).  It is correct but slow; the block (MHFFNLayer.heads_and_gate) does not route that case to it.
+ALLOWED_SCRATCH = ("mhffn_gate_bwd_kernelILi128ELi2ELb1E",)
+
+
 def check_no_scratch(usage):
     """The hand-scheduled kernels assume every value stays in registers: a spill would put VALU copies of matrix results
-    into places the explicit wait states do not cover.  Fails the build if the compiler reports private (scratch)
-    memory for one of them."""
+    into places the explicit wait states do not cover, and in the bandwidth-bound head prologue it multiplies the
+    run time.  Fails the build if the compiler reports private (scratch) memory for one of them, and also if the
+    resource remarks of an expected kernel are missing (a changed remark format must not pass silently)."""
+    for frag, count in EXPECTED_KERNELS:
+        found = [n for n in usage if frag in n and "ScratchSize" in usage[n]]
+        if len(found) != count:
+            raise RuntimeError(f"expected resource-usage remarks for {count} instantiations of {frag}, found {len(found)}")
     for name, u in usage.items():
-        if ("mhffn_fwd_kernel" in name or "mhffn_bwd_" in name) and int(u.get("ScratchSize", "0")) != 0:
+        if any(frag in name for frag, _ in EXPECTED_KERNELS) and int(u["ScratchSize"]) != 0:
+            if any(a in name for a in ALLOWED_SCRATCH):
+                continue
             raise RuntimeError(f"{name} uses {u['ScratchSize']} bytes of scratch per lane: a spill in a hand-scheduled kernel")
 
 

@@ -67,7 +67,8 @@ const char* mhffn_strerror(int code)
         case MHFFN_ERR_DTYPE: return "unsupported dtype (Q, K, U, V must all be bfloat16 or all float32; R float32)";
         case MHFFN_ERR_HEAD_DIM: return "unsupported head dim (bf16: d_h must be 64, 96 or 128; fp32: a multiple of 8 up to 128)";
         case MHFFN_ERR_EXPERT_DIM: return "unsupported expert dim (bf16: d_e must be a multiple of 32)";
-        case MHFFN_ERR_SHAPE: return "invalid extents (all must be positive, H a multiple of Hkuv; bf16: E <= 64)";
+        case MHFFN_ERR_SHAPE:
+            return "invalid extents (all must be positive, H a multiple of Hkuv; bf16: E <= 64), token layout or phase mask";
         case MHFFN_ERR_WORKSPACE: return "workspace missing or too small";
         case MHFFN_ERR_LAUNCH: return "kernel launch failed";
         case MHFFN_ERR_ALIGNMENT: return "pointer not 16-byte aligned";
@@ -107,6 +108,7 @@ int mhffn_fwd_layout(const void* Q, const void* K, const void* U, const void* V,
     const int rc = check_dims_impl(dims, dtype);
     if (rc != MHFFN_OK) return rc;
     if (token_layout != MHFFN_TOKENS_BHSD && token_layout != MHFFN_TOKENS_BSHD) return MHFFN_ERR_SHAPE;
+    if (phases & ~MHFFN_FWD_ALL) return MHFFN_ERR_SHAPE;       // a bit this build does not define: refuse, do not ignore
     if (!Q || !K || !U || !V || !R || !O) return MHFFN_ERR_NULL_POINTER;
     if (!aligned16(Q) || !aligned16(K) || !aligned16(U) || !aligned16(V) || !aligned16(R) || !aligned16(O) ||
         !aligned16(workspace))
@@ -144,6 +146,7 @@ int mhffn_bwd_layout(const void* Q, const void* K, const void* U, const void* V,
     if (rc != MHFFN_OK) return rc;
     if (token_layout != MHFFN_TOKENS_BHSD && token_layout != MHFFN_TOKENS_BSHD) return MHFFN_ERR_SHAPE;
     if (grad_w_dtype != MHFFN_DTYPE_BF16 && grad_w_dtype != MHFFN_DTYPE_F32) return MHFFN_ERR_DTYPE;
+    if (phases & ~MHFFN_BWD_ALL) return MHFFN_ERR_SHAPE;       // a bit this build does not define: refuse, do not ignore
     if (!Q || !K || !U || !V || !R || !dO || !dQ || !dK || !dU || !dV || !dR) return MHFFN_ERR_NULL_POINTER;
     const void* ptrs[] = {Q, K, U, V, R, dO, dQ, dK, dU, dV, dR, workspace};
     for (const void* p : ptrs)

@@ -160,7 +160,8 @@ __global__ __launch_bounds__(256) void mhffn_gate_fwd_kernel(GateArgs p)
     constexpr int KS = DH / 16;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float* sW = reinterpret_cast<float*>(smem + 2 * NT * KS * 1024);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, g = lane >> 5;
+    const int lane = threadIdx.x & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     float* rtile = sW + DH + wave * (TILE_B / 4);
     const int h = blockIdx.y, b = blockIdx.z;
 
@@ -217,12 +218,14 @@ constexpr size_t gate_bwd_smem(int DH, int NT)
            4 * 128 * 4;
 }
 
-template <int CT>
-__device__ __forceinline__ bf16x8 tile_cols(const unsigned char* tile, const TrLane<CT>& tl, int ct, int s)
+// Transposed operand (column tile ct, k-half s) of a swizzled tile.  Only column tile 0's two lane offsets are kept in
+// registers: the swizzle XORs the chunk index, and a column tile is 4 chunks = 64 bytes, so tile ct's offset is tile
+// 0's with bits 6..7 XORed by ct (one VALU instruction per read instead of two more registers per column tile).
+__device__ __forceinline__ bf16x8 tile_cols(const unsigned char* tile, const TrLane<1>& tl, int ct, int s)
 {
     typedef __attribute__((address_space(3))) v4bf16_t* lds_v4;
-    const v4bf16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4)(tile + tl.off[ct][0] + 4096 * s));
-    const v4bf16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4)(tile + tl.off[ct][1] + 4096 * s));
+    const v4bf16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4)(tile + (tl.off[0][0] ^ (ct << 6)) + 4096 * s));
+    const v4bf16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4)(tile + (tl.off[0][1] ^ (ct << 6)) + 4096 * s));
     bf16x8 r;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -240,7 +243,8 @@ __global__ __launch_bounds__(256) void mhffn_gate_bwd_kernel(GateArgs p)
     unsigned char* sA = smem;                                   // logits operands
     unsigned char* sC = sA + 2 * NT * KS * 1024;                // dy operands
     float* sW = reinterpret_cast<float*>(sC + CT * 2 * NT * 1024);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, g = lane >> 5;
+    const int lane = threadIdx.x & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: tile counters and tile bases stay scalar
     unsigned char* regions = reinterpret_cast<unsigned char*>(sW + DH);
     unsigned char* ytile = regions + wave * GATE_WAVE_REGION_B;
     unsigned char* ztile = ytile + TILE_B;
@@ -254,7 +258,7 @@ __global__ __launch_bounds__(256) void mhffn_gate_bwd_kernel(GateArgs p)
     // they are written as zeros every tile, so nothing needs clearing here
     __syncthreads();
 
-    const TrLane<CT> trl = make_tr_lane<CT, 8, 4>(lane);
+    const TrLane<1> trl = make_tr_lane<1, 8, 4>(lane);
     const TokRows dqrows = tok_rows(p.dq_tokmaj, b, h, p.H, p.S);
     f32x16 wacc[CT][NT];            // d_router partial: rows = columns of y, cols = experts
     float dwacc[KS][8];             // d_norm_weight partial for the lane's own columns
@@ -409,10 +413,10 @@ __global__ __launch_bounds__(256) void mhffn_gate_bwd_kernel(GateArgs p)
         for (int s = 0; s < 2; ++s) {
             bf16x8 bz[NT];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) bz[nt] = tile_cols<CT>(ztile, trl, nt, s);
+            for (int nt = 0; nt < NT; ++nt) bz[nt] = tile_cols(ztile, trl, nt, s);
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                const bf16x8 ay = tile_cols<CT>(ytile, trl, ct, s);
+                const bf16x8 ay = tile_cols(ytile, trl, ct, s);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) wacc[ct][nt] = mfma32(ay, bz[nt], wacc[ct][nt]);
             }

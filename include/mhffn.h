@@ -68,7 +68,9 @@ int mhffn_is_supported(int d_h, int d_e, int dtype);
 /* Checks extents and dtype only (no pointers, no GPU).  Returns MHFFN_OK or the error the launch would return. */
 int mhffn_check_dims(const mhffn_dims* dims, int dtype);
 
-/* Scratch bytes needed by mhffn_fwd / mhffn_bwd for these extents (0 on invalid extents). */
+/* Scratch bytes needed by mhffn_fwd / mhffn_bwd for these extents.  0 is a valid answer, not only the answer for invalid
+ * extents (ask mhffn_check_dims for those): the forward never needs scratch, and the bfloat16 backward needs none where
+ * its dK/dU/dV kernel runs as one token slice (e.g. the 370M and 1.3B layers); `workspace` may then be NULL. */
 size_t mhffn_fwd_workspace_bytes(const mhffn_dims* dims, int dtype);
 size_t mhffn_bwd_workspace_bytes(const mhffn_dims* dims, int dtype);
 
@@ -96,7 +98,8 @@ int mhffn_bwd(const void* Q, const void* K, const void* U, const void* V, const 
  * earlier full call with the same arguments has filled.  mhffn_fwd == mhffn_fwd_phases(..., MHFFN_FWD_ALL) and
  * mhffn_bwd == mhffn_bwd_phases(..., MHFFN_BWD_ALL).  They exist so a benchmark can bracket one kernel with HIP
  * events on the launch stream; the reference has no counterpart (its kernels are launched one per Python call,
- * flash_mlp_moe.py:832-866). */
+ * flash_mlp_moe.py:832-866).  A mask with a bit outside MHFFN_FWD_ALL / MHFFN_BWD_ALL returns MHFFN_ERR_SHAPE (the bit
+ * values are not stable across versions of this header: pass the names, not numbers). */
 enum {
     MHFFN_FWD_MAIN = 1, MHFFN_FWD_ALL = 1,
     MHFFN_BWD_DQDR = 1, MHFFN_BWD_DKDUDV = 2, MHFFN_BWD_REDUCE = 4, MHFFN_BWD_ALL = 7

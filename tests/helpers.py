@@ -19,3 +19,32 @@ def make_inputs(B, H, S, dh, E, de, Hk=None, *, seed=0, dtype=torch.float32, r_m
     cast = lambda t: t.to(dtype).to(device)
     R = R.to(torch.float64 if dtype == torch.float64 else torch.float32)
     return cast(Q), cast(K), cast(U), cast(V), R.to(device), cast(dO)
+
+
+# bf16 parity bars: max-abs <= 2e-2 and mean-rel <= 1e-2.
+# O, dQ and dR do not grow with the number of tokens and are held to the max-abs bar as a raw figure -- O and dQ while
+# they can meet it at all: they are stored in bf16, whose spacing above |v| = 4 is 1/32 or more, so where max|ref|
+# exceeds 4 (single-expert shapes, whose gate is 1 instead of about 1/E; the reference script's unnormalised N(0,1) gate)
+# the bar is taken relative to max|ref| / 4.  dR is stored in fp32: raw everywhere.
+# dK, dU and dV are sums over all tokens (|dK| ~ sqrt(tokens): 45 at the 370M layer's 16,384 tokens, where one bf16 ulp is
+# 0.25 and the rounding of the bf16 matrix operands alone random-walks past 2e-2): their max-abs bar is relative to
+# max(1, max|ref|), the figure the reference's script prints (kernels/thunderkittens/run_from_python.py:54-58), and
+# tests/test_gpu_parity_bars.py holds them, at the benchmark's sizes, to "no further from the fp64 gradients than the
+# reference's own eager path run in bf16".
+MAX_ABS, MEAN_REL = 2e-2, 1e-2
+
+
+def assert_bf16_parity(name, got, ref, context=None):
+    from oracle import mhffn_oracle as orc
+    m = orc.error_metrics(got, ref)
+    peak = ref.abs().max().item()
+    if name == "dR":
+        scale = 1.0
+    elif name in ("O", "dQ"):
+        scale = max(1.0, peak / 4.0)
+    else:
+        scale = max(1.0, peak)
+    assert torch.isfinite(got).all(), (name, context)
+    assert m["max_abs"] <= MAX_ABS * scale, (name, context, m, f"bar scaled by {scale}")
+    assert m["mean_rel"] <= MEAN_REL or ref.abs().sum().item() < 1e-3, (name, context, m)
+    return m

@@ -95,10 +95,15 @@ def test_entry_points_validate_before_touching_the_gpu(L):
     bad = _capi.Dims(1, 2, 2, 64, 128, 2, 65)
     assert L.mhffn_fwd(ok, ok, ok, ok, ok, ok, ok, 1 << 30, bad, 0, null) == _capi.ERR_EXPERT_DIM
     # token-layout variants: same checks, plus the layout code itself
-    assert L.mhffn_fwd_layout(null, null, null, null, null, null, null, 0, d, 0, _capi.TOKENS_BSHD, null, 3) == _capi.ERR_NULL_POINTER
-    assert L.mhffn_fwd_layout(ok, ok, ok, ok, ok, ok, ok, 1 << 30, d, 0, 7, null, 3) == _capi.ERR_SHAPE
-    assert L.mhffn_bwd_layout(*([ok] * 11), 0, ok, 1 << 30, d, 0, -1, null, 15) == _capi.ERR_SHAPE
-    assert L.mhffn_bwd_layout(*([ok] * 11), 0, ok, 16, sliced, 0, _capi.TOKENS_BSHD, null, 15) == _capi.ERR_WORKSPACE
+    assert L.mhffn_fwd_layout(null, null, null, null, null, null, null, 0, d, 0, _capi.TOKENS_BSHD, null, _capi.FWD_ALL) == _capi.ERR_NULL_POINTER
+    assert L.mhffn_fwd_layout(ok, ok, ok, ok, ok, ok, ok, 1 << 30, d, 0, 7, null, _capi.FWD_ALL) == _capi.ERR_SHAPE
+    assert L.mhffn_bwd_layout(*([ok] * 11), 0, ok, 1 << 30, d, 0, -1, null, _capi.BWD_ALL) == _capi.ERR_SHAPE
+    assert L.mhffn_bwd_layout(*([ok] * 11), 0, ok, 16, sliced, 0, _capi.TOKENS_BSHD, null, _capi.BWD_ALL) == _capi.ERR_WORKSPACE
+    # phase masks with a bit the header does not define are refused, not ignored (the bit values have changed before)
+    assert L.mhffn_fwd_layout(ok, ok, ok, ok, ok, ok, ok, 1 << 30, d, 0, 0, null, 2) == _capi.ERR_SHAPE
+    assert L.mhffn_fwd_phases(ok, ok, ok, ok, ok, ok, ok, 1 << 30, d, 0, null, 3) == _capi.ERR_SHAPE
+    assert L.mhffn_bwd_layout(*([ok] * 11), 0, ok, 1 << 30, d, 0, 0, null, 8) == _capi.ERR_SHAPE
+    assert L.mhffn_bwd_phases(*([ok] * 11), 0, ok, 1 << 30, d, 0, null, 15) == _capi.ERR_SHAPE
     # more than 2^31 token rows are rejected (row indices are 32-bit inside the kernels)
     huge = _capi.Dims(4096, 64, 64, 1 << 14, 128, 2, 64)
     assert L.mhffn_check_dims(huge, 0) == _capi.ERR_SHAPE

@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from oracle import mhffn_oracle as orc
+from tests.helpers import assert_bf16_parity
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 FILES = sorted(glob.glob(os.path.join(HERE, "golden", "*.npz")))
@@ -48,6 +49,4 @@ def test_hip_kernels_match_golden(path):
     grads = mhffn_backward(*ins, g["dO"].to(torch.bfloat16).to(dev), grad_w_dtype=torch.float32)
     torch.cuda.synchronize()
     for name, got in zip(("O",) + NAMES, (O,) + tuple(grads)):
-        m = orc.error_metrics(got.float().cpu(), g[name])
-        scale = max(1.0, g[name].abs().max().item())
-        assert m["max_abs"] <= 2e-2 * scale and m["mean_rel"] <= 1e-2, (name, m)
+        assert_bf16_parity(name, got.float().cpu(), g[name], os.path.basename(path))

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import mhffn_oracle as orc
-from tests.helpers import make_inputs
+from tests.helpers import assert_bf16_parity, make_inputs
 
 pytestmark = pytest.mark.gpu
 
@@ -33,9 +33,4 @@ def test_edge_shapes_match_oracle(B, H, S, dh, E, de, Hk):
     g = mhffn_backward(*ins, dO.to(dev), grad_w_dtype=torch.float32)
     torch.cuda.synchronize()
     for name, got, ref in zip(("O", "dQ", "dK", "dU", "dV", "dR"), (O,) + tuple(g), (ref_O,) + tuple(ref_g)):
-        assert torch.isfinite(got).all(), name
-        m = orc.error_metrics(got.float().cpu(), ref.float())
-        scale = max(1.0, ref.abs().max().item())
-        print(name, m, flush=True)
-        assert m["max_abs"] <= 2e-2 * scale, (name, m)
-        assert m["mean_rel"] <= 1e-2 or ref.abs().sum() < 1e-3, (name, m)
+        print(name, assert_bf16_parity(name, got.float().cpu(), ref.float()), flush=True)

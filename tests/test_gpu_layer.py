@@ -1,7 +1,8 @@
 """The MH-FFN block on the GPU (HIP operator, token-major Q/O, bf16) against the fp32 CPU restatement of the reference
 module (oracle.mhffn_block_forward, models/flashmhf/modeling_mhffnmoe.py:352-431) with the same parameters: the block
 output and the gradients of the input x (dX), of K, U, V and of the router.  Bars as for the operator: mean-rel 1e-2,
-max-abs 2e-2 relative to the quantity's scale."""
+max-abs 2e-2 relative to the quantity's scale; the router's gradient and the decoder's embedding gradient must in addition
+be no worse than what the same block gives with the reference's bf16 eager operator."""
 import pytest
 import torch
 
@@ -58,8 +59,28 @@ def test_block_forward_backward_matches_fp32_restatement(B, S, hid, H, Hk, E, de
     for n in ("K", "U", "V"):
         _check(getattr(layer, n).grad, ref_leaves[n].grad, "d" + n)
     rname = "router" if router_input == "q" else "w_router"
-    # the gate gradient passes through dR (a d_e-long sum of bf16 products): its bar is looser in the mean
-    _check(getattr(layer, rname).grad, ref_leaves[rname].grad, "d" + rname, mean_rel=3e-2)
+    # The gate's gradient sums dR * dgate over all tokens, with dR a d_e-long sum of products of bf16-rounded factors.
+    # Its bar is the operator's (mean-rel 1e-2, max-abs 2e-2 of its scale), and it must also be no further from the fp32
+    # restatement than the reference's own block in bf16 is -- the same parameters with the eager expert loop
+    # (models/flashmhf/modeling_mhffnmoe.py:412-431) and the torch prologue.
+    hip = orc.error_metrics(getattr(layer, rname).grad.float().cpu(), ref_leaves[rname].grad)
+    eager_layer = MHFFNLayer(hid, H, E, de, Hk, apply_rmsnorm=rms, router_input=router_input, op=_EagerBf16(),
+                             fused_prologue=False).to(dev).to(torch.bfloat16)
+    eager_layer.load_state_dict(layer.state_dict())
+    xe = x.to(dev).requires_grad_(True)
+    eager_layer(xe).backward(g.to(dev))
+    torch.cuda.synchronize()
+    eag = orc.error_metrics(getattr(eager_layer, rname).grad.float().cpu(), ref_leaves[rname].grad)
+    print("d" + rname, "HIP", hip, "bf16 eager block", eag, flush=True)
+    assert hip["norm_max"] <= 2e-2 and hip["mean_rel"] <= 1e-2, hip
+    assert hip["mean_rel"] <= eag["mean_rel"], (hip, eag)
+
+
+class _EagerBf16(torch.nn.Module):
+    """The reference's eager expert loop in the tensors' own dtype (bf16), differentiated by torch.autograd."""
+
+    def forward(self, Q, K, U, V, R):
+        return orc.mhffn_forward(Q, K, U, V, R, compute_dtype=Q.dtype, out_dtype=Q.dtype)
 
 
 def test_small_decoder_step_matches_the_same_model_on_the_eager_operator():
@@ -84,11 +105,23 @@ def test_small_decoder_step_matches_the_same_model_on_the_eager_operator():
     loss_ref = model(ids, labels=ids)
     loss_ref.backward()
     torch.cuda.synchronize()
-    print("loss", loss.item(), loss_ref.item(), flush=True)
+    g_ref = model.embed.weight.grad.float().clone()
+    # third run: the operator as the reference's eager loop in bf16 -- what a bf16 model without the fused kernel gives
+    model.zero_grad()
+    for blk in model.blocks:
+        blk.mlp.op = _EagerBf16()
+    loss_eager = model(ids, labels=ids)
+    loss_eager.backward()
+    torch.cuda.synchronize()
+    print("loss", loss.item(), loss_ref.item(), loss_eager.item(), flush=True)
     assert torch.isfinite(loss) and abs(loss.item() - loss_ref.item()) <= 2e-2 * abs(loss_ref.item())
-    m = orc.error_metrics(g_hip.cpu(), model.embed.weight.grad.float().cpu())
-    print("embed grad", m, flush=True)
-    assert m["mean_rel"] <= 5e-2
+    m = orc.error_metrics(g_hip.cpu(), g_ref.cpu())
+    me = orc.error_metrics(model.embed.weight.grad.float().cpu(), g_ref.cpu())
+    print("embed grad: HIP operator", m, "bf16 eager operator", me, flush=True)
+    # Two bf16 decoder blocks, attention included, sit between the operator and this gradient.  Bar: the operator's
+    # mean-rel 1e-2, and no further from the fp32-operator gradient than the same model is when only the operator is
+    # swapped for the reference's bf16 eager loop (with a quarter of slack: both figures are one sample of rounding noise).
+    assert m["mean_rel"] <= 1e-2 and m["mean_rel"] <= 1.25 * me["mean_rel"], (m, me)
 
 
 def test_legacy_single_expert_operator_is_a_per_head_swiglu():
@@ -142,3 +175,42 @@ def test_fused_block_norm_stays_within_the_second_rounding_of_the_reference_form
         norm.weight.fill_(1.0)
         ulp1 = 2.0 ** (torch.floor(torch.log2(normed.float().abs().clamp(min=1e-30))) - 7)
         assert ((norm(x).float() - normed.float()).abs() <= ulp1).all()
+
+
+def test_many_experts_with_head_norm_at_width_128_takes_the_torch_prologue(monkeypatch):
+    """d_h = 128 with more than 32 experts and per-head RMSNorm: the fused prologue's backward kernel for that
+    combination does not fit the register file, so the block keeps the torch prologue there (and only there), and
+    its results still match the fp32 restatement."""
+    import flashmhf_amd.mhffn_layer as ml
+    calls = []
+    real = ml.head_norm_gate
+    monkeypatch.setattr(ml, "head_norm_gate", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    torch.manual_seed(5)
+    B, S, H, E, de = 2, 100, 2, 40, 32
+    hid = H * 128
+    for rms, expect_fused in ((True, False), (False, True)):
+        calls.clear()
+        layer = MHFFNLayer(hid, H, E, de, apply_rmsnorm=rms)
+        with torch.no_grad():
+            layer.w_self.weight.normal_(std=hid ** -0.5)
+            layer.w_self_2.weight.normal_(std=hid ** -0.5)
+        layer = layer.to(torch.bfloat16)
+        x = torch.randn(B, S, hid).to(torch.bfloat16)
+        g = torch.randn(B, S, hid).to(torch.bfloat16)
+        ref_leaves = {n: p.detach().float().requires_grad_(True) for n, p in layer.named_parameters()}
+        x_ref = x.float().requires_grad_(True)
+        y_ref = orc.mhffn_block_forward(x_ref, ref_leaves["w_self.weight"], ref_leaves["w_self_2.weight"], ref_leaves["K"],
+                                        ref_leaves["U"], ref_leaves["V"], num_heads=H, router=ref_leaves["router"],
+                                        q_norm_weight=ref_leaves.get("q_norm.weight"))
+        y_ref.backward(g.float())
+        layer = layer.to("cuda:0")
+        xg = x.to("cuda:0").requires_grad_(True)
+        y = layer(xg)
+        y.backward(g.to("cuda:0"))
+        torch.cuda.synchronize()
+        assert bool(calls) == expect_fused, (rms, calls)
+        _check(y, y_ref.detach(), "Y")
+        _check(xg.grad, x_ref.grad, "dX")
+        m = orc.error_metrics(layer.router.grad.float().cpu(), ref_leaves["router"].grad)
+        print("rms", rms, "d_router", m, flush=True)
+        assert m["norm_max"] <= 2e-2 and m["mean_rel"] <= 1e-2, m

@@ -5,6 +5,7 @@ import pytest
 import torch
 
 from oracle import mhffn_oracle as orc
+from tests.helpers import assert_bf16_parity
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -44,8 +45,7 @@ def test_1p3b_layer_rows_match_oracle_and_weight_gradients_add_over_batch():
     ref_O = orc.mhffn_forward(sub(Q), Kc, Uc, Vc, sub(R), compute_dtype=torch.float32)
     ref = orc.mhffn_backward(sub(Q), Kc, Uc, Vc, sub(R), sub(dO), compute_dtype=torch.float64)
     for name, got, r in (("O", sub(O), ref_O), ("dQ", sub(dQ), ref[0]), ("dR", sub(dR), ref[4])):
-        m = orc.error_metrics(got.float(), r)
-        assert m["max_abs"] <= 2e-2 * max(1.0, r.abs().max().item()) and m["mean_rel"] <= 1e-2, (name, m)
+        assert_bf16_parity(name, got.float(), r)          # raw max-abs 2e-2, mean-rel 1e-2
     # dK, dU, dV are sums over tokens: the whole batch equals the sum of its elements run one by one (fp32 partial sums
     # are added in a different order, hence a tolerance instead of equality)
     acc = [torch.zeros_like(dK) for _ in range(3)]

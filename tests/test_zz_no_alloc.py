@@ -84,3 +84,28 @@ def test_static_scratch_backward_rejects_what_does_not_fit_before_any_launch():
     assert rc == _capi.ERR_STATIC_SCRATCH
     assert "mhffn_bwd_static" in _capi.strerror(rc)
     assert L.mhffn_bwd_workspace_bytes(dims, _capi.DTYPE_F32) > _capi.STATIC_SCRATCH_BYTES
+
+
+def test_static_scratch_backward_allocates_no_device_memory():
+    """The property the entry point exists for: after one warm-up call (address look-up, LDS opt-in) a call changes
+    neither the device's free memory nor torch's allocator statistics.  Problem with several token slices, so the fixed
+    array is really used."""
+    from flashmhf_amd import _capi
+    L = _capi.lib()
+    B, H, S, dh, E, de, Hk = 2, 4, 1024, 128, 8, 256, 4
+    Q, K, U, V, R, dO = (t.to(DEV) for t in make_inputs(B, H, S, dh, E, de, Hk, seed=5, dtype=torch.bfloat16))
+    dims = _capi.Dims(B, H, Hk, S, dh, E, de)
+    assert L.mhffn_bwd_workspace_bytes(dims, 0) > 0
+    outs = [torch.empty_like(Q), *(torch.empty_like(K) for _ in range(3)), torch.empty_like(R)]
+    st = torch.cuda.current_stream().cuda_stream
+    args = (*(t.data_ptr() for t in (Q, K, U, V, R, dO)), *(t.data_ptr() for t in outs), 0, dims, 0, 0, st)
+    assert L.mhffn_bwd_static(*args) == 0
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    reserved0, allocated0 = torch.cuda.memory_reserved(), torch.cuda.memory_allocated()
+    for _ in range(3):
+        assert L.mhffn_bwd_static(*args) == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, (free0, free1)
+    assert (torch.cuda.memory_reserved(), torch.cuda.memory_allocated()) == (reserved0, allocated0)
