@@ -40,7 +40,6 @@ __global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
 {
     constexpr int KS = DH / 16, CT = DH / 32, NW = 8;
     constexpr int BT = NW * 32;
-    constexpr int NTHR = NW * 64;
     constexpr int FILL = 24 / NW;          // tile-fill wave-instructions per wave and block (3 tiles x 8 / NW waves)
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     float* sR = reinterpret_cast<float*>(smem + DQ_NST * DQ_STAGE_B);   // [E][BT]
@@ -68,9 +67,7 @@ __global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
             tile_fill_ins<DH>(Kh + toff + roff, DH, st + which * TILE_B, id & 7, lane);
         }
     };
-    issue_block(0);
-    issue_block(1);
-
+    // The Q and dO rows come from HBM and are the longest wait of the prologue: request them before anything else.
     bf16x8 q[KS], go[KS];
     {
         int t = tok0 + l32;
@@ -83,11 +80,18 @@ __global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
             go[ks] = *reinterpret_cast<const bf16x8*>(gr + ks * 16);
         }
     }
-    for (int idx = tid; idx < BT * p.E; idx += NTHR) {
-        int t = tb * BT + idx / p.E;
+    issue_block(0);
+    // Gate values of the workgroup's 256 tokens, expert-major [E][BT]: asynchronous 4-byte LDS-direct loads, lane = token;
+    // a pair of waves shares a group of 64 tokens and takes the even and the odd experts.  Issued between block 0 and
+    // block 1, so that the first wait for block 0 covers them too.
+    {
+        int t = tb * BT + (wave >> 1) * 64 + lane;
         t = t < p.S ? t : p.S - 1;
-        sR[(idx % p.E) * BT + idx / p.E] = p.R[(rowbase + t) * p.E + idx % p.E];
+        const float* rrow = p.R + (rowbase + t) * p.E;
+        for (int e = wave & 1; e < p.E; e += 2)
+            __builtin_amdgcn_global_load_lds((gptr_t)(rrow + e), (lptr_t)(sR + e * BT + (wave >> 1) * 64), 4, 0, 0);
     }
+    issue_block(1);
 
     f32x16 dq[CT];
 #pragma unroll
@@ -172,21 +176,32 @@ __global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
             if (g == 0 && t < p.S) p.dR[(rowbase + t) * p.E + e] = tot;
         }
     }
-    wait_vmcnt<0>();   // drain the phantom prefetches before the workgroup's LDS is released
+    wait_vmcnt<0>();   // drain the phantom prefetches: they write the ring, which the epilogue reuses
+    __syncthreads();   // every wave is done reading the ring
 
+    // dQ^T registers -> dQ[t][c] through a private 8 KB region of the ring per wave (rows of 256 bytes, 16-byte chunk c16
+    // of row r at chunk c16 ^ (r & 15)), so that the stores are whole rows (16 lanes x 16 bytes, 4 rows per instruction)
+    // instead of 8-byte pieces scattered over 32 rows.  Register 4a+x of row tile i is c = 32i + 8a + 4g + x.
     {
-        const int t = tok0 + l32;
-        if (t < p.S) {
-            bf16_t* orow = p.dQ + (qrows.base + (long)t * qrows.stride) * DH;
+        unsigned char* otile = smem + wave * (32 * TILE_ROW_B);
 #pragma unroll
-            for (int i = 0; i < CT; ++i)
+        for (int i = 0; i < CT; ++i)
 #pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    bf16x4 v;
+            for (int a = 0; a < 4; ++a) {
+                bf16x4 v;
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) v[x] = (bf16_t)dq[i][4 * a + x];
-                    *reinterpret_cast<bf16x4*>(orow + 32 * i + 8 * a + 4 * g) = v;
-                }
+                for (int x = 0; x < 4; ++x) v[x] = (bf16_t)dq[i][4 * a + x];
+                *reinterpret_cast<bf16x4*>(otile + l32 * TILE_ROW_B + (((4 * i + a) ^ (l32 & 15)) << 4) + 8 * g) = v;
+            }
+        const int c16 = lane & 15;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int row = 4 * k + (lane >> 4);
+            const int t = tok0 + row;
+            if (c16 < DH / 8 && t < p.S) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(otile + row * TILE_ROW_B + ((c16 ^ (row & 15)) << 4));
+                *reinterpret_cast<u32x4*>(p.dQ + (qrows.base + (long)t * qrows.stride) * DH + c16 * 8) = v;
+            }
         }
     }
 }
@@ -350,6 +365,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
             }
         }
         wait_vmcnt<0>();
+        __syncthreads();   // the barrier the working waves pass before their epilogue reuses the ring
         return;
     }
 
@@ -573,54 +589,70 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         }
     }
     wait_vmcnt<0>();
+    __syncthreads();      // every wave is done reading the tile ring, which the epilogue reuses
 
+    // dK^T registers 4a+x of row tile ct: c = 32ct + 8a + 4g + x, column j = l32, i.e. a lane owns runs of 4 c of weight row
+    // j.  Stored directly these are 8- or 16-byte pieces scattered over 32 rows per instruction; instead each wave passes
+    // one gradient block at a time through a private 16 KB region of the ring (16-byte chunk c16 of row r at chunk
+    // c16 ^ r), reads it back row-wise and stores whole rows.  Only this wave touches the region, and LDS operations of
+    // one wave complete in order, so no barrier is needed between the three blocks.
     {
-        // dK^T registers 4a+b of row tile ct: c = 32ct + 8a + 4g + b, column j = l32 -> runs of 4 along c.
+        unsigned char* region = smem_raw + wave * 16384;
         const long wsz = (long)gridDim.x * nblk * JB * DH;   // elements of one weight tensor
+        const long row0 = (wrow - l32) * DH;                 // first element of this wave's block of rows
+        auto store_f32 = [&](const f32x16 (&acc)[CT], float* dst) {      // rows of DH floats, 512-byte rows in LDS
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    f32x4 v;
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) v[x] = acc[ct][4 * a + x];
+                    *reinterpret_cast<f32x4*>(region + l32 * 512 + (((8 * ct + 2 * a + g) ^ l32) << 4)) = v;
+                }
+            const int c16 = lane & 31;
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                const int row = 2 * k + (lane >> 5);
+                if (c16 < DH / 4) {
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(region + row * 512 + ((c16 ^ row) << 4));
+                    *reinterpret_cast<u32x4*>(dst + row0 + row * DH + c16 * 4) = v;
+                }
+            }
+        };
+        auto store_bf16 = [&](const f32x16 (&acc)[CT], bf16_t* dst) {    // rows of DH bf16, 256-byte rows in LDS
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    bf16x4 v;
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) v[x] = (bf16_t)acc[ct][4 * a + x];
+                    *reinterpret_cast<bf16x4*>(region + l32 * 256 + (((4 * ct + a) ^ (l32 & 15)) << 4) + 8 * g) = v;
+                }
+            const int c16 = lane & 15;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int row = 4 * k + (lane >> 4);
+                if (c16 < DH / 8) {
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(region + row * 256 + ((c16 ^ (row & 15)) << 4));
+                    *reinterpret_cast<u32x4*>(dst + row0 + row * DH + c16 * 8) = v;
+                }
+            }
+        };
         if (p.nslice > 1) {                                  // fp32 partial sums of this token slice
-            float* base = p.part + (long)z * 3 * wsz + wrow * DH;
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    const int c = 32 * ct + 8 * a + 4 * g;
-                    f32x4 v0, v1, v2;
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) { v0[x] = dk[ct][4 * a + x]; v1[x] = du[ct][4 * a + x]; v2[x] = dv[ct][4 * a + x]; }
-                    *reinterpret_cast<f32x4*>(base + c) = v0;
-                    *reinterpret_cast<f32x4*>(base + wsz + c) = v1;
-                    *reinterpret_cast<f32x4*>(base + 2 * wsz + c) = v2;
-                }
+            float* base = p.part + (long)z * 3 * wsz;
+            store_f32(dk, base);
+            store_f32(du, base + wsz);
+            store_f32(dv, base + 2 * wsz);
         } else if (p.out_f32) {                              // one slice: the sums are the gradients
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    const long o = wrow * DH + 32 * ct + 8 * a + 4 * g;
-                    f32x4 v0, v1, v2;
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) { v0[x] = dk[ct][4 * a + x]; v1[x] = du[ct][4 * a + x]; v2[x] = dv[ct][4 * a + x]; }
-                    *reinterpret_cast<f32x4*>(static_cast<float*>(p.out[0]) + o) = v0;
-                    *reinterpret_cast<f32x4*>(static_cast<float*>(p.out[1]) + o) = v1;
-                    *reinterpret_cast<f32x4*>(static_cast<float*>(p.out[2]) + o) = v2;
-                }
+            store_f32(dk, static_cast<float*>(p.out[0]));
+            store_f32(du, static_cast<float*>(p.out[1]));
+            store_f32(dv, static_cast<float*>(p.out[2]));
         } else {
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    const long o = wrow * DH + 32 * ct + 8 * a + 4 * g;
-                    bf16x4 v0, v1, v2;
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        v0[x] = (bf16_t)dk[ct][4 * a + x];
-                        v1[x] = (bf16_t)du[ct][4 * a + x];
-                        v2[x] = (bf16_t)dv[ct][4 * a + x];
-                    }
-                    *reinterpret_cast<bf16x4*>(static_cast<bf16_t*>(p.out[0]) + o) = v0;
-                    *reinterpret_cast<bf16x4*>(static_cast<bf16_t*>(p.out[1]) + o) = v1;
-                    *reinterpret_cast<bf16x4*>(static_cast<bf16_t*>(p.out[2]) + o) = v2;
-                }
+            store_bf16(dk, static_cast<bf16_t*>(p.out[0]));
+            store_bf16(du, static_cast<bf16_t*>(p.out[1]));
+            store_bf16(dv, static_cast<bf16_t*>(p.out[2]));
         }
     }
 }

@@ -46,7 +46,7 @@ constexpr int FWD_RING_B = 3 * FWD_REGION_B;     // 96 KB
 template <int DH>
 __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
 {
-    constexpr int KS = DH / 16, CT = DH / 32, NW = 4, BT = NW * 64, NTHR = NW * 64;
+    constexpr int KS = DH / 16, CT = DH / 32, NW = 4, BT = NW * 64;
     constexpr int FILL = 24 / NW;
     constexpr int NG1 = 4 * KS, NG2 = 4 * CT, NSLOT = NG1 + NG2;   // MFMAs per step
     // The first products of a step are written by inline-assembly MFMAs whose results the next step's element-wise code
@@ -80,10 +80,7 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
             tile_fill_ins<DH>(Kh + toff + roff, DH, smem + region + stage * TILE_B, id & 7, lane);
         }
     };
-    issue_block(0, 0);
-    issue_block(1, 1);
-    issue_block(2, 2);
-
+    // The Q rows come from HBM and are the longest wait of the prologue: request them before anything else.
     bf16x8 q[2][KS];
 #pragma unroll
     for (int ct = 0; ct < 2; ++ct) {
@@ -93,11 +90,20 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) q[ct][ks] = *reinterpret_cast<const bf16x8*>(qr + ks * 16);
     }
-    for (int idx = tid; idx < BT * p.E; idx += NTHR) {
-        int t = tb * BT + idx / p.E;
+    issue_block(0, 0);
+    // Gate values of the workgroup's 256 tokens, expert-major [E][BT]: one asynchronous 4-byte LDS-direct load per expert
+    // and wave (lane = token, so the 64 values of an instruction are contiguous in LDS).  Issued between block 0 and
+    // block 1, so that the wait for block 0 below covers them too.
+    {
+        int t = tok0 + lane;
         t = t < p.S ? t : p.S - 1;
-        sR[(idx % p.E) * BT + idx / p.E] = p.R[(rowbase + t) * p.E + idx % p.E];
+        const float* rrow = p.R + (rowbase + t) * p.E;
+        for (int e = 0; e < p.E; ++e)
+            __builtin_amdgcn_global_load_lds((gptr_t)(rrow + e), (lptr_t)(sR + e * BT + wave * 64), 4, 0, 0);
     }
+    issue_block(1, 1);
+    issue_block(2, 2);
+
 
     f32x16 oacc[CT][2];
 #pragma unroll
@@ -214,7 +220,7 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     };
 
     f32x16 mA[2], nA[2], mB[2], nB[2];
-    wait_vmcnt<2 * FILL>();   // block 0 (and the Q / R loads before it) have landed
+    wait_vmcnt<2 * FILL>();   // all but the fills of blocks 1 and 2: block 0 and the gate values have landed
     __syncthreads();
     {
 #pragma unroll
@@ -258,14 +264,18 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
             if (blk + 2 < nblk) step(S2{}, blk + 2, e, mA, nA, mB, nB);
         }
     }
-    wait_vmcnt<0>();      // drain the phantom prefetches before the workgroup's LDS is released
+    wait_vmcnt<0>();      // drain the phantom prefetches: they write the ring, which the epilogue reuses
+    __syncthreads();      // every wave is done reading the ring
 
-    // O^T registers -> O[t][c]: register 4a+b of row tile i is c = 32i + 8a + 4g + b, so each lane owns runs of 4 c.
+    // O^T registers -> O[t][c].  Register 4a+b of row tile i is c = 32i + 8a + 4g + b: a lane owns runs of 4 c of one
+    // token, which stored directly would be 8-byte pieces scattered over 32 rows per instruction.  Instead each wave
+    // writes its 64 x d_h tile into a private 16 KB region of the ring (rows of 256 bytes, 16-byte chunk c16 of row r at
+    // chunk c16 ^ (r & 15)), reads it back row-wise and stores whole rows: 16 lanes x 16 bytes per row, 4 rows per
+    // instruction.  Only this wave touches the region, and LDS operations of one wave complete in order.
+    {
+        unsigned char* otile = smem + wave * (64 * TILE_ROW_B);
 #pragma unroll
-    for (int ct = 0; ct < 2; ++ct) {
-        const int t = tok0 + ct * 32 + l32;
-        if (t < p.S) {
-            bf16_t* orow = p.O + (qrows.base + (long)t * qrows.stride) * DH;
+        for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
             for (int i = 0; i < CT; ++i)
 #pragma unroll
@@ -273,8 +283,17 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
                     bf16x4 v;
 #pragma unroll
                     for (int x = 0; x < 4; ++x) v[x] = (bf16_t)oacc[i][ct][4 * a + x];
-                    *reinterpret_cast<bf16x4*>(orow + 32 * i + 8 * a + 4 * g) = v;
+                    *reinterpret_cast<bf16x4*>(otile + (ct * 32 + l32) * TILE_ROW_B + (((4 * i + a) ^ (l32 & 15)) << 4) + 8 * g) = v;
                 }
+        const int c16 = lane & 15;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const int row = 4 * k + (lane >> 4);
+            const int t = tok0 + row;
+            if (c16 < DH / 8 && t < p.S) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(otile + row * TILE_ROW_B + ((c16 ^ (row & 15)) << 4));
+                *reinterpret_cast<u32x4*>(p.O + (qrows.base + (long)t * qrows.stride) * DH + c16 * 8) = v;
+            }
         }
     }
 }
