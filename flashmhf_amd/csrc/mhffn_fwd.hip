@@ -104,7 +104,6 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     issue_block(1, 1);
     issue_block(2, 2);
 
-
     f32x16 oacc[CT][2];
 #pragma unroll
     for (int i = 0; i < CT; ++i)
@@ -133,12 +132,12 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
         issue_block(blk + 3, (ST + 3) % FWD_NST);
 
         // The gate value enters through its reciprocal: r / (1 + e) = 1 / fma(e, 1/r, 1/r), one multiply fewer per
-        // element.  1/r is clamped to the largest finite float, so r = 0 (a zero gate, or the phantom block behind an odd
-        // count) makes the denominator at least FLT_MAX, whose reciprocal the hardware flushes to exactly 0.
+        // element.  1/r is clamped to the largest finite float, so a zero gate makes the denominator at least FLT_MAX, whose
+        // reciprocal the hardware flushes to exactly 0.
         float rinv[2];
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) {
-            const float rv = blk < nblk ? sR[(e < p.E ? e : p.E - 1) * BT + wave * 64 + ct * 32 + l32] : 0.0f;
+            const float rv = sR[e * BT + wave * 64 + ct * 32 + l32];
             rinv[ct] = __builtin_amdgcn_fmed3f(__builtin_amdgcn_rcpf(rv), -FLT_MAX_F, FLT_MAX_F);
         }
         auto read_k = [&](int ks) { return *reinterpret_cast<const bf16x8*>(kbase[ks] + STN * TILE_B); };
