@@ -7,7 +7,7 @@ any bf16 implementation.  For them the criterion is the one the reference's own 
 (kernels/thunderkittens/run_from_python.py:40-58 compares the kernel with the eager path): the HIP gradients must be
 no further from the fp64 gradients than the reference's eager expert loop run in bf16 under torch.autograd
 (models/flashmhf/modeling_mhffnmoe.py:412-431) is, in raw max-abs and in mean-rel, and mean-rel <= 1e-2 as stated.
-The raw figures are printed (pytest -s) and recorded in BASELINE.md.
+The raw figures are printed (pytest -s).
 """
 import pytest
 import torch
