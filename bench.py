@@ -197,12 +197,14 @@ def device_state_under(fn, seconds=0.5):
     return out
 
 
-def measured_mfma_peak_tflops(dev):
-    """Rate of a register-resident v_mfma_f32_32x32x16_bf16 loop on every SIMD (mhffn_probe_mfma_peak), ~5 ms per launch."""
+def measured_mfma_peak_tflops(dev, random_data=False):
+    """Rate of a register-resident v_mfma_f32_32x32x16_bf16 loop on every SIMD (mhffn_probe_mfma_loop), ~5 ms per launch.
+    random_data: operand values in which every bit varies (as in real activations and weights) instead of small, smoothly
+    varying ones; the package grants a lower clock for them."""
     import ctypes
     from flashmhf_amd import build as b
     L = ctypes.CDLL(b.PROBE_LIB)
-    L.mhffn_probe_mfma_peak.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+    L.mhffn_probe_mfma_loop.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                         ctypes.POINTER(ctypes.c_double)]
     sink = torch.zeros(4, device=dev)
     flops = ctypes.c_double(0.0)
@@ -210,7 +212,7 @@ def measured_mfma_peak_tflops(dev):
     st = torch.cuda.current_stream().cuda_stream
 
     def run():
-        rc = L.mhffn_probe_mfma_peak(sink.data_ptr(), blocks, 10000, st, ctypes.byref(flops))
+        rc = L.mhffn_probe_mfma_loop(sink.data_ptr(), blocks, 10000, int(random_data), st, ctypes.byref(flops))
         assert rc == 0, rc
 
     ms = time_events(run, 5, warm=3)
@@ -641,6 +643,7 @@ def run_workload(name, args, dev, light=False):
 
     kt, kstate = kernel_timings(w, ins, sample_state=not light)
     mfma_loop, probe_state = (None, None) if light else measured_mfma_peak_tflops(dev)
+    mfma_loop_rnd, probe_state_rnd = (None, None) if light else measured_mfma_peak_tflops(dev, random_data=True)
     dom = max(CREDIT, key=lambda k: kt.get(k, 0.0))
     ach = CREDIT[dom] * f1(w) / (kt[dom] * 1e-3) / 1e12
     traffic, traffic_note = recorded_traffic(name, dom)
@@ -663,6 +666,8 @@ def run_workload(name, args, dev, light=False):
         "frac_of_mfma_peak": tflops / PEAK_BF16_TFLOPS,
         "measured_mfma_loop_tflops": mfma_loop,
         "measured_mfma_loop_under_load": probe_state,
+        "measured_mfma_loop_random_operands_tflops": mfma_loop_rnd,
+        "measured_mfma_loop_random_operands_under_load": probe_state_rnd,
         "nominal_peak_clock_mhz": 2400,
         "frac_of_measured_mfma_loop": tflops / mfma_loop if mfma_loop else None,
         "tokens_per_s": tokens / (ms * 1e-3),
