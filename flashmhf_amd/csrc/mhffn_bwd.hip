@@ -42,7 +42,7 @@ __global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
     constexpr int BT = NW * 32;
     constexpr int FILL = 24 / NW;          // tile-fill wave-instructions per wave and block (3 tiles x 8 / NW waves)
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-    float* sR = reinterpret_cast<float*>(smem + DQ_NST * DQ_STAGE_B);   // [E][BT]
+    float* sR = reinterpret_cast<float*>(smem + DQ_NST * DQ_STAGE_B);   // [min(E, GATE_WIN)][BT]: one expert window
 
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -82,15 +82,21 @@ __global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
     }
     issue_block(0);
     // Gate values of the workgroup's 256 tokens, expert-major [E][BT]: asynchronous 4-byte LDS-direct loads, lane = token;
-    // a pair of waves shares a group of 64 tokens and takes the even and the odd experts.  Issued between block 0 and
-    // block 1, so that the first wait for block 0 covers them too.
+    // a pair of waves shares a group of 64 tokens and takes the even and the odd experts.  LDS holds a window of GATE_WIN
+    // experts at a time; the first is issued between block 0 and block 1, so that the first wait for block 0 covers it
+    // too, and a layer with more experts restages the tile at the top of the expert loop.
+    const float* rrow;
     {
         int t = tb * BT + (wave >> 1) * 64 + lane;
         t = t < p.S ? t : p.S - 1;
-        const float* rrow = p.R + (rowbase + t) * p.E;
-        for (int e = wave & 1; e < p.E; e += 2)
-            __builtin_amdgcn_global_load_lds((gptr_t)(rrow + e), (lptr_t)(sR + e * BT + (wave >> 1) * 64), 4, 0, 0);
+        rrow = p.R + (rowbase + t) * p.E;
     }
+    auto stage_gates = [&](int e0) {
+        const int e1 = e0 + GATE_WIN < p.E ? e0 + GATE_WIN : p.E;
+        for (int e = e0 + (wave & 1); e < e1; e += 2)
+            __builtin_amdgcn_global_load_lds((gptr_t)(rrow + e), (lptr_t)(sR + (e - e0) * BT + (wave >> 1) * 64), 4, 0, 0);
+    };
+    stage_gates(0);
     issue_block(1);
 
     f32x16 dq[CT];
@@ -103,6 +109,12 @@ __global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
     const TrLane<CT> trl = make_tr_lane<CT, 8, 4>(lane);
     int blk = 0;
     for (int e = 0; e < p.E; ++e) {
+        if (e > 0 && (e & (GATE_WIN - 1)) == 0) {
+            __syncthreads();      // every wave has read its gate values of the window before
+            stage_gates(e);
+            wait_vmcnt<0>();      // (also lands the blocks in flight; the next wait for a block then passes at once)
+            __syncthreads();
+        }
         float dr = 0.0f;
         for (int jb = 0; jb < p.nbe; ++jb, ++blk) {
             wait_vmcnt<FILL>();       // block blk has landed (block blk+1 may be in flight)
@@ -112,19 +124,34 @@ __global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
             const unsigned char* sK = smem + (blk % DQ_NST) * DQ_STAGE_B;
             const unsigned char* sU = sK + TILE_B;
             const unsigned char* sV = sU + TILE_B;
-            const float r = sR[e * BT + wave * 32 + l32];
+            const float r = sR[(e & (GATE_WIN - 1)) * BT + wave * 32 + l32];
 
             f32x16 m, n, da;
 #pragma unroll
             for (int x = 0; x < 16; ++x) { m[x] = 0.0f; n[x] = 0.0f; da[x] = 0.0f; }
+            {
+                // The K/U/V operands come from LDS through a ring of three register sets, read two k-steps ahead of the
+                // matrix instructions that use them; the fence after each k-step keeps the compiler from gathering the
+                // reads back to the front (which costs their whole latency once per block).
+                bf16x8 ak[3], au[3], av[3];
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8 ak = tile_read_rows(sK, krow, ks, g);
-                const bf16x8 au = tile_read_rows(sU, krow, ks, g);
-                const bf16x8 av = tile_read_rows(sV, krow, ks, g);
-                m = mfma32(ak, q[ks], m);
-                n = mfma32(au, q[ks], n);
-                da = mfma32(av, go[ks], da);
+                for (int k0 = 0; k0 < 2; ++k0) {
+                    ak[k0] = tile_read_rows(sK, krow, k0, g);
+                    au[k0] = tile_read_rows(sU, krow, k0, g);
+                    av[k0] = tile_read_rows(sV, krow, k0, g);
+                }
+                static_for<KS>([&](auto kc) {
+                    constexpr int ks = decltype(kc)::value;
+                    if constexpr (ks + 2 < KS) {
+                        ak[(ks + 2) % 3] = tile_read_rows(sK, krow, ks + 2, g);
+                        au[(ks + 2) % 3] = tile_read_rows(sU, krow, ks + 2, g);
+                        av[(ks + 2) % 3] = tile_read_rows(sV, krow, ks + 2, g);
+                    }
+                    m = mfma32(ak[ks % 3], q[ks], m);
+                    n = mfma32(au[ks % 3], q[ks], n);
+                    da = mfma32(av[ks % 3], go[ks], da);
+                    __builtin_amdgcn_sched_barrier(0);
+                });
             }
 
             bf16x8 dmt[2], dnt[2];
@@ -726,7 +753,7 @@ static hipError_t launch_bwd_t(const void* Q, const void* K, const void* U, cons
         DqArgs a{(const bf16_t*)Q, (const bf16_t*)dO, (const bf16_t*)K, (const bf16_t*)U, (const bf16_t*)V, R,
                  (bf16_t*)dQ, dR, d.H, G, d.S, d.E, nbe, d.tokmaj};
         const int tokw = 256;
-        const int smem = DQ_NST * DQ_STAGE_B + d.E * tokw * (int)sizeof(float);
+        const int smem = DQ_NST * DQ_STAGE_B + (d.E < GATE_WIN ? d.E : GATE_WIN) * tokw * (int)sizeof(float);
         if (smem > 160 * 1024) return hipErrorInvalidValue;
         static LdsOptIn optin;
         err = ensure_dynamic_lds(optin, (const void*)mhffn_bwd_dqdr_kernel<DH>, smem);

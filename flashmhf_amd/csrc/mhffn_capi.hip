@@ -21,7 +21,6 @@ int check_dims_impl(const mhffn_dims* d, int dtype)
     if (dtype == MHFFN_DTYPE_F32) {           // fp32 correctness path: generic tiles, no MFMA
         if (d->d_h % 8 != 0 || d->d_h > 128) return MHFFN_ERR_HEAD_DIM;
     } else {
-        if (d->E > 64) return MHFFN_ERR_SHAPE;   // the kernels stage a [E][256] fp32 gate tile in LDS next to the weight ring
         if (d->d_h != 64 && d->d_h != 96 && d->d_h != 128) return MHFFN_ERR_HEAD_DIM;
         if (d->d_e % 32 != 0) return MHFFN_ERR_EXPERT_DIM;
     }
@@ -68,7 +67,7 @@ const char* mhffn_strerror(int code)
         case MHFFN_ERR_HEAD_DIM: return "unsupported head dim (bf16: d_h must be 64, 96 or 128; fp32: a multiple of 8 up to 128)";
         case MHFFN_ERR_EXPERT_DIM: return "unsupported expert dim (bf16: d_e must be a multiple of 32)";
         case MHFFN_ERR_SHAPE:
-            return "invalid extents (all must be positive, H a multiple of Hkuv; bf16: E <= 64), token layout or phase mask";
+            return "invalid extents (all must be positive, H a multiple of Hkuv; gate kernels: E <= 64), token layout or phase mask";
         case MHFFN_ERR_WORKSPACE: return "workspace missing or too small";
         case MHFFN_ERR_LAUNCH: return "kernel launch failed";
         case MHFFN_ERR_ALIGNMENT: return "pointer not 16-byte aligned";

@@ -30,6 +30,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // 16-byte copy unit (native vector: stays in registers)
 
 constexpr int JB = 32;          // rows of K/U/V per block
+// Experts whose gate values the forward and the dQ/dR kernel keep in LDS at a time ([GATE_WIN][256 tokens] fp32 = 64 KB,
+// next to the 96 KB weight ring); a power of two, and a window is a multiple of four blocks whatever d_e is.
+constexpr int GATE_WIN = 64;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float FLT_MAX_F = 3.402823466e+38f;
 

@@ -54,7 +54,7 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     // what covers the 18 wait states an MFMA result needs before a VALU read.
     static_assert(NG2 >= 8, "the second-product MFMAs of a step must cover the hazard window of its first products");
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-    float* sR = reinterpret_cast<float*>(smem + FWD_RING_B);   // [E][BT]
+    float* sR = reinterpret_cast<float*>(smem + FWD_RING_B);   // [min(E, GATE_WIN)][BT]: gate values of one expert window
 
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -92,15 +92,21 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     }
     issue_block(0, 0);
     // Gate values of the workgroup's 256 tokens, expert-major [E][BT]: one asynchronous 4-byte LDS-direct load per expert
-    // and wave (lane = token, so the 64 values of an instruction are contiguous in LDS).  Issued between block 0 and
-    // block 1, so that the wait for block 0 below covers them too.
+    // and wave (lane = token, so the 64 values of an instruction are contiguous in LDS).  LDS holds a window of GATE_WIN
+    // experts at a time; the first window is issued between block 0 and block 1, so that the wait for block 0 below
+    // covers it too, and a layer with more experts restages the tile between two steps of the block loop.
+    const float* rrow;
     {
         int t = tok0 + lane;
         t = t < p.S ? t : p.S - 1;
-        const float* rrow = p.R + (rowbase + t) * p.E;
-        for (int e = 0; e < p.E; ++e)
-            __builtin_amdgcn_global_load_lds((gptr_t)(rrow + e), (lptr_t)(sR + e * BT + wave * 64), 4, 0, 0);
+        rrow = p.R + (rowbase + t) * p.E;
     }
+    auto stage_gates = [&](int e0) {
+        const int e1 = e0 + GATE_WIN < p.E ? e0 + GATE_WIN : p.E;
+        for (int e = e0; e < e1; ++e)
+            __builtin_amdgcn_global_load_lds((gptr_t)(rrow + e), (lptr_t)(sR + (e - e0) * BT + wave * 64), 4, 0, 0);
+    };
+    stage_gates(0);
     issue_block(1, 1);
     issue_block(2, 2);
 
@@ -137,7 +143,7 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
         float rinv[2];
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) {
-            const float rv = sR[e * BT + wave * 64 + ct * 32 + l32];
+            const float rv = sR[(e & (GATE_WIN - 1)) * BT + wave * 64 + ct * 32 + l32];
             rinv[ct] = __builtin_amdgcn_fmed3f(__builtin_amdgcn_rcpf(rv), -FLT_MAX_F, FLT_MAX_F);
         }
         auto read_k = [&](int ks) { return *reinterpret_cast<const bf16x8*>(kbase[ks] + STN * TILE_B); };
@@ -244,15 +250,25 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     auto advance = [&]() {
         if (++jb == p.nbe) { jb = 0; ++e; }
     };
-    for (; blk + 4 <= nblk; blk += 4) {
-        step(S0{}, blk, e, mA, nA, mB, nB);
-        advance();
-        step(S1{}, blk + 1, e, mB, nB, mA, nA);
-        advance();
-        step(S2{}, blk + 2, e, mA, nA, mB, nB);
-        advance();
-        step(S3{}, blk + 3, e, mB, nB, mA, nA);
-        advance();
+    // (A window of GATE_WIN experts is a multiple of four blocks, so every window starts on stage 0 and register set A.)
+    for (int e0 = 0; e0 < p.E; e0 += GATE_WIN) {
+        if (e0 > 0) {
+            __syncthreads();      // every wave has read its gate values of the window before
+            stage_gates(e0);
+            wait_vmcnt<0>();      // (also lands the two blocks in flight; the next step's wait then passes at once)
+            __syncthreads();
+        }
+        const int wend = (e0 + GATE_WIN) * p.nbe < nblk ? (e0 + GATE_WIN) * p.nbe : nblk;
+        for (; blk + 4 <= wend; blk += 4) {
+            step(S0{}, blk, e, mA, nA, mB, nB);
+            advance();
+            step(S1{}, blk + 1, e, mB, nB, mA, nA);
+            advance();
+            step(S2{}, blk + 2, e, mA, nA, mB, nB);
+            advance();
+            step(S3{}, blk + 3, e, mB, nB, mA, nA);
+            advance();
+        }
     }
     if (blk < nblk) {
         step(S0{}, blk, e, mA, nA, mB, nB);
@@ -301,7 +317,7 @@ template <int DH>
 static hipError_t launch_fwd_t(const FwdArgs& a, const Dims& d, hipStream_t st)
 {
     const int tokw = 256;
-    const int smem = FWD_RING_B + d.E * tokw * (int)sizeof(float);
+    const int smem = FWD_RING_B + (d.E < GATE_WIN ? d.E : GATE_WIN) * tokw * (int)sizeof(float);
     if (smem > 160 * 1024) return hipErrorInvalidValue;
     static LdsOptIn optin;
     const hipError_t e = ensure_dynamic_lds(optin, (const void*)mhffn_fwd_kernel<DH>, smem);

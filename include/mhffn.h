@@ -39,7 +39,7 @@ enum {
     MHFFN_ERR_DTYPE        = -2,  /* reference: TypeError, flash_mlp_moe.py:761-766; TORCH_CHECK flash_ffn_moe.cu:943-945 */
     MHFFN_ERR_HEAD_DIM     = -3,  /* reference: assert head_dim == 128, flash_ffn_moe.cu:956 */
     MHFFN_ERR_EXPERT_DIM   = -4,  /* reference: ValueError, flash_mlp_moe.py:758-759; assert flash_ffn_moe.cu:958 */
-    MHFFN_ERR_SHAPE        = -5,  /* non-positive extent, H not a multiple of Hkuv, bf16 with E > 64 */
+    MHFFN_ERR_SHAPE        = -5,  /* non-positive extent, H not a multiple of Hkuv, gate kernels with E > 64 */
     MHFFN_ERR_WORKSPACE    = -6,  /* workspace missing or smaller than *_workspace_bytes() */
     MHFFN_ERR_LAUNCH       = -7,  /* hipGetLastError() after a launch */
     MHFFN_ERR_ALIGNMENT    = -8,  /* a tensor or workspace pointer is not 16-byte aligned */
@@ -60,7 +60,7 @@ typedef struct mhffn_dims {
 /* Human-readable text for a return code (static storage). */
 const char* mhffn_strerror(int code);
 
-/* 1 if kernels exist for (d_h, d_e, dtype), else 0.  bf16 (MFMA kernels): d_h in {64, 96, 128}, d_e % 32 == 0, E <= 64.
+/* 1 if kernels exist for (d_h, d_e, dtype), else 0.  bf16 (MFMA kernels): d_h in {64, 96, 128}, d_e % 32 == 0, any E.
  * float32 (correctness instantiation, plain FMA): d_h a multiple of 8 up to 128, any d_e, any E.
  * Replaces the reference's shape gates (flash_mlp_moe.py:758, flash_ffn_moe.cu:956-958, 1037). */
 int mhffn_is_supported(int d_h, int d_e, int dtype);

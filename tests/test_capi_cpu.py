@@ -51,7 +51,7 @@ def test_strerror_and_is_supported(L):
     ((8, 8, 8, 2048, 100, 11, 352), 0, _capi.ERR_HEAD_DIM),
     ((8, 8, 3, 2048, 128, 11, 352), 0, _capi.ERR_SHAPE),
     ((0, 8, 8, 2048, 128, 11, 352), 0, _capi.ERR_SHAPE),
-    ((8, 8, 8, 2048, 128, 65, 352), 0, _capi.ERR_SHAPE),
+    ((8, 8, 8, 2048, 128, 65, 352), 0, _capi.OK),            # more experts than one LDS gate window holds
     ((8, 8, 8, 2048, 128, 11, 352), 1, 0),
     ((8, 8, 8, 2048, 100, 11, 352), 1, _capi.ERR_HEAD_DIM),
     ((8, 8, 8, 2048, 128, 11, 352), 7, _capi.ERR_DTYPE),

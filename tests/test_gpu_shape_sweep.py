@@ -1,6 +1,6 @@
 """Seeded sweep over shapes the fixed cases do not visit: ragged sequence lengths around the 32/64/256-token tile
 boundaries, odd and even counts of 32-row blocks per expert (the forward's phantom block, the dK/dU/dV tail
-instantiation), grouped K/U/V heads with every divisor, expert counts up to the limit of 64, all three head widths,
+instantiation), grouped K/U/V heads with every divisor, expert counts up to and beyond one LDS gate window of 64, all three head widths,
 both token layouts and both weight-gradient dtypes.  Every case: forward and all five gradients against the fp64 oracle
 on the same bf16-rounded inputs, at the bars of the fixed cases (mean-rel 1e-2; max-abs 2e-2 raw for O, dQ, dR and relative to
 max(1, max|ref|) for dK, dU, dV: tests/helpers.py)."""
@@ -59,6 +59,22 @@ def test_forward_and_backward_match_the_oracle_over_the_sweep(case):
     for name, got, ref in zip(("O", "dQ", "dK", "dU", "dV", "dR"), (O,) + tuple(g), (ref_O,) + tuple(ref_g)):
         assert got.shape == ref.shape, (name, case)
         _check(got.float().cpu(), ref, name, case)
+
+
+# More experts than the 64 whose gate values the forward and the dQ/dR kernel hold in LDS at a time: one expert past a
+# window, exactly two windows, windows that end inside the four-block trips of the forward (d_e = 64: two blocks per
+# expert), three windows with a ragged last one.
+CASES_MANY_EXPERTS = [
+    (1, 2, 300, 128, 65, 32, 1, False, "bf16"),
+    (2, 1, 257, 64, 128, 32, 1, True, "f32"),
+    (1, 2, 513, 96, 130, 64, 2, False, "bf16"),
+    (1, 1, 64, 128, 200, 32, 1, True, "bf16"),
+]
+
+
+@pytest.mark.parametrize("case", CASES_MANY_EXPERTS, ids=["B{}H{}S{}dh{}E{}de{}Hk{}{}{}".format(*c[:7], "tm" if c[7] else "hm", c[8]) for c in CASES_MANY_EXPERTS])
+def test_more_experts_than_one_gate_window(case):
+    test_forward_and_backward_match_the_oracle_over_the_sweep(case)
 
 
 def _cases_f32(n=20, seed=77):
