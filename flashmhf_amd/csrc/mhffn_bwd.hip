@@ -414,8 +414,9 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
 
     const int fr = swz16(l32);
     const TrLane<CT> trl = make_tr_lane<CT, 4, 8>(lane);
-    const int rowoff = l32 * 256;
-    const int xg = (g ^ fr) << 4;                     // chunk byte offset of k-step 0; k-step ks is xg ^ (ks << 5)
+    // LDS address of this lane's 16 bytes of k-step 0 in the Q tile of stage 0 (row l32, chunk g ^ swizzle); k-step ks is
+    // this address ^ (ks << 5): the ring starts on a 1 KB boundary, so the exclusive-or commutes with the sum
+    const unsigned qaddr = lds_addr(smem_raw) + l32 * 256 + ((g ^ fr) << 4);
 
     // first products of the tile in stage ST -> (m, n, da) in architectural VGPRs, element-wise work of the PREVIOUS
     // tile (registers pm, pn, pda; gate values from stage SP) dealt out between the k-steps so that the VALU works
@@ -433,17 +434,39 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         const float* pR = live ? reinterpret_cast<const float*>(pG + TILE_B) + wave * 64 : sZero;
 
         bf16x8 pB[2], dmB[2], dnB[2];
-        bf16x8 aq[3], ag[3];                         // operand ring: k-step ks+2 is requested while ks is consumed
-#pragma unroll
-        for (int k0 = 0; k0 < 2; ++k0) {
-            const int off = rowoff + (xg ^ (k0 << 5));
-            aq[k0] = *reinterpret_cast<const bf16x8*>(sQ + off);
-            ag[k0] = *reinterpret_cast<const bf16x8*>(sG + off);
+        // LDS reads of the first products: the gate values of the previous tile for this lane's 16 token rows (4
+        // consecutive rows per 16-byte read), then the operand ring (k-step ks + 2 is requested while ks is consumed).
+        // All are issued from inline assembly and waited for by count; the element-wise slices in between are VALU only.
+        __builtin_amdgcn_sched_barrier(0);
+        u32x4 rvu[4];
+        {
+            const unsigned ra = lds_addr(pR) + 16 * g;
+            rvu[0] = lds_read16_async<0>(ra);
+            rvu[1] = lds_read16_async<32>(ra);
+            rvu[2] = lds_read16_async<64>(ra);
+            rvu[3] = lds_read16_async<96>(ra);
         }
-        // gate values of the previous tile for this lane's 16 token rows (4 consecutive rows per 16-byte read)
+        u32x4 aq[3], ag[3];
+        auto request = [&](auto kc) {
+            constexpr int ks = decltype(kc)::value;
+            const unsigned a = qaddr ^ (ks << 5);     // the stage goes into the instruction's immediate offset
+            aq[ks % 3] = lds_read16_async<ST * DW_STAGE_B>(a);
+            ag[ks % 3] = lds_read16_async<ST * DW_STAGE_B + TILE_B>(a);
+        };
+        request(std::integral_constant<int, 0>{});
+        request(std::integral_constant<int, 1>{});
         f32x4 rv[4];
-#pragma unroll
-        for (int a = 0; a < 4; ++a) rv[a] = *reinterpret_cast<const f32x4*>(pR + 8 * a + 4 * g);
+        // Transposed operands of the token contraction (phases 2 and 3 below), in (s, ct) order.  They come from the
+        // previous tile, so the first two sets are requested under the last two k-steps of the first products, in the
+        // ring slots those no longer need, and have arrived when the contraction starts.
+        constexpr int NSET = 2 * CT;
+        TrOperand tq[3], tg[3];
+        auto request_tr = [&](auto ic) {
+            constexpr int idx = decltype(ic)::value;
+            constexpr int s = idx / CT, ct = idx % CT;
+            tq[idx % 3] = tile_read_cols_async<4096 * s>(lds_addr(pQ), trl, ct);
+            tg[idx % 3] = tile_read_cols_async<4096 * s + TILE_B>(lds_addr(pQ), trl, ct);
+        };
 
         // Element-wise work of the previous tile, two elements (register indices 2pr, 2pr+1 of pm/pn/pda) at a time so
         // that no instruction waits on the one just before it, in five slices of at most six VALU instructions; one slice
@@ -497,19 +520,27 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         };
         static_for<KS>([&](auto kc) {
             constexpr int ks = decltype(kc)::value;
-            if constexpr (ks + 2 < KS) {
-                const int off = rowoff + (xg ^ ((ks + 2) << 5));
-                aq[(ks + 2) % 3] = *reinterpret_cast<const bf16x8*>(sQ + off);
-                ag[(ks + 2) % 3] = *reinterpret_cast<const bf16x8*>(sG + off);
+            if constexpr (ks + 2 < KS) request(std::integral_constant<int, ks + 2>{});
+            if constexpr (ks == KS - 2) request_tr(std::integral_constant<int, 0>{});
+            if constexpr (ks == KS - 1) request_tr(std::integral_constant<int, 1>{});
+            // reads younger than this k-step's operands: two per later k-step of the ring, four per transposed set
+            constexpr int younger = ks + 2 < KS ? 4 : (ks == KS - 2 ? 2 + 4 : 4 + 4);
+            if constexpr (ks == 0) {
+                lds_wait_n<younger>(aq[0], ag[0], rvu[0], rvu[1], rvu[2], rvu[3]);       // (the gate values are older)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) rv[a] = __builtin_bit_cast(f32x4, rvu[a]);
+            } else {
+                lds_wait_n<younger>(aq[ks % 3], ag[ks % 3]);
             }
-            if constexpr (ks == 0) mfma32_vgpr_first_bacc(m, aq[0], kB[0]);
-            else mfma32_vgpr_acc_bacc(m, aq[ks % 3], kB[ks]);
+            const bf16x8 aqv = __builtin_bit_cast(bf16x8, aq[ks % 3]), agv = __builtin_bit_cast(bf16x8, ag[ks % 3]);
+            if constexpr (ks == 0) mfma32_vgpr_first_bacc(m, aqv, kB[0]);
+            else mfma32_vgpr_acc_bacc(m, aqv, kB[ks]);
             after_slot1(std::integral_constant<int, 3 * ks>{});
-            if constexpr (ks == 0) mfma32_vgpr_first_bacc(n, aq[0], uB[0]);
-            else mfma32_vgpr_acc_bacc(n, aq[ks % 3], uB[ks]);
+            if constexpr (ks == 0) mfma32_vgpr_first_bacc(n, aqv, uB[0]);
+            else mfma32_vgpr_acc_bacc(n, aqv, uB[ks]);
             after_slot1(std::integral_constant<int, 3 * ks + 1>{});
-            if constexpr (ks == 0) mfma32_vgpr_first(da, ag[0], vR[0]);
-            else mfma32_vgpr_acc(da, ag[ks % 3], vR[ks]);
+            if constexpr (ks == 0) mfma32_vgpr_first(da, agv, vR[0]);
+            else mfma32_vgpr_acc(da, agv, vR[ks]);
             after_slot1(std::integral_constant<int, 3 * ks + 2>{});
         });
 
@@ -520,20 +551,10 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         // LDS instruction, so the partial LDS waits count exactly the asynchronous reads.
         __builtin_amdgcn_sched_barrier(0);
         {
-            constexpr int NSET = 2 * CT;              // (s, ct) in s-major order
-            TrOperand tq[3], tg[3];
-            auto request = [&](auto ic) {
-                constexpr int idx = decltype(ic)::value;
-                constexpr int s = idx / CT, ct = idx % CT;
-                tq[idx % 3] = tile_read_cols_async<4096 * s>(lds_addr(pQ), trl, ct);
-                tg[idx % 3] = tile_read_cols_async<4096 * s + TILE_B>(lds_addr(pQ), trl, ct);
-            };
-            request(std::integral_constant<int, 0>{});
-            request(std::integral_constant<int, 1>{});
             static_for<NSET>([&](auto ic) {
                 constexpr int idx = decltype(ic)::value;
                 constexpr int s = idx / CT, ct = idx % CT;
-                if constexpr (idx + 2 < NSET) request(std::integral_constant<int, idx + 2>{});
+                if constexpr (idx + 2 < NSET) request_tr(std::integral_constant<int, idx + 2>{});
                 constexpr int ahead = (NSET - 1 - idx) < 2 ? (NSET - 1 - idx) : 2;
                 lds_tr_wait_n<4 * ahead>(tq[idx % 3], tg[idx % 3]);
                 // s = 0: list 2 is dealt out over the 3 CT MFMAs of this half
@@ -560,7 +581,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         // issued since then cover the wait states before the next step's element-wise code reads them; what is still
         // needed is that their registers stay allocated to the end of the step even when nothing reads them (the
         // phantom steps), or the compiler hands them to other values that the late write would overwrite.
-        static_assert(6 * CT >= 8, "the contraction MFMAs of a step must cover the hazard window of its first products");
+        static_assert(KS >= 2 && NSET >= 2 && 6 * CT >= 8, "the contraction MFMAs of a step must cover the hazard window of its first products");
         asm volatile("" :: "v"(m), "v"(n), "v"(da));
     };
 

@@ -230,6 +230,28 @@ __device__ __forceinline__ void lds_tr_wait_n(TrOperand& a, TrOperand& b)
 {
     asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a.lo), "+v"(a.hi), "+v"(b.lo), "+v"(b.hi) : "n"(N));
 }
+// The same for 16 contiguous bytes per lane (a row-major A operand as in tile_read_rows, four gate values): issued from
+// inline assembly so that the waits in front of the uses can be partial -- the compiler's own bookkeeping puts a full
+// lgkmcnt(0) in front of the first use of any read of a group in flight.  IMM: compile-time displacement.
+template <int IMM>
+__device__ __forceinline__ u32x4 lds_read16_async(unsigned addr)
+{
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(IMM));
+    return v;
+}
+// At most N LDS operations of this wave still outstanding; the operands cannot be used above it.  Same conditions as
+// lds_tr_wait_n.
+template <int N>
+__device__ __forceinline__ void lds_wait_n(u32x4& a, u32x4& b)
+{
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_n(u32x4& a, u32x4& b, u32x4& c, u32x4& d, u32x4& e, u32x4& f)
+{
+    asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f) : "n"(N));
+}
 __device__ __forceinline__ bf16x8 tr_value(const TrOperand& t)
 {
     u32x4 v = {t.lo[0], t.lo[1], t.hi[0], t.hi[1]};
