@@ -423,7 +423,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     // under the MFMAs; then the token contraction of the previous tile.
     //   registers 4a+b of m/n/da: token 8a + 4g + b (rows), column j = l32.
     auto step = [&](auto st_c, auto sp_c, f32x16& m, f32x16& n, f32x16& da, const f32x16& pm, const f32x16& pn,
-                    const f32x16& pda, bool live) {
+                    const f32x16& pda, bool live, int& nv_next) {
         constexpr int ST = decltype(st_c)::value, SP = decltype(sp_c)::value;
         const unsigned char* sQ = smem_raw + ST * DW_STAGE_B;
         const unsigned char* sG = sQ + TILE_B;
@@ -455,6 +455,11 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         };
         request(std::integral_constant<int, 0>{});
         request(std::integral_constant<int, 1>{});
+        // The fill of the stage that came free at the barrier (tile k + 2) is issued behind the first reads: its five
+        // instructions and their address arithmetic pass while those reads are on their way.
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (TAIL) prepare_tile();     // (the tail instantiation has no registers to spare for the early call)
+        nv_next = fire_tile((ST + 2) % DW_NST);
         f32x4 rv[4];
         // Transposed operands of the token contraction (phases 2 and 3 below), in (s, ct) order.  They come from the
         // previous tile, so the first two sets are requested under the last two k-steps of the first products, in the
@@ -592,7 +597,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     f32x16 mA, nA, dA_, mB, nB, dB_;
 #pragma unroll
     for (int x = 0; x < 16; ++x) { mA[x] = 0.0f; nA[x] = 0.0f; dA_[x] = 0.0f; mB[x] = 0.0f; nB[x] = 0.0f; dB_[x] = 0.0f; }
-    auto sync_step = [&](auto st_c, int nvalid, int& nv_next) {
+    auto sync_step = [&](auto st_c, int nvalid) {
         constexpr int ST = decltype(st_c)::value;
         // All of this wave's loads, not only the older tile's: a partial count (the next tile's loads still in flight)
         // measured no faster.
@@ -603,8 +608,6 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         // (a bare barrier: the LDS-direct loads were waited for just above, and this wave's LDS reads of the stage that
         // is refilled next were consumed by the matrix instructions of the step before)
         __builtin_amdgcn_s_barrier();
-        if constexpr (TAIL) prepare_tile();     // (the tail instantiation has no registers to spare for the early call)
-        nv_next = fire_tile((ST + 2) % DW_NST);
     };
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
@@ -614,24 +617,24 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     {
         int k = 0;
         for (; k + 3 <= nt; k += 4) {
-            sync_step(I0{}, nv0, nv2);
-            step(I0{}, I3{}, mA, nA, dA_, mB, nB, dB_, k > 0);
-            sync_step(I1{}, nv1, nv3);
-            step(I1{}, I0{}, mB, nB, dB_, mA, nA, dA_, true);
-            sync_step(I2{}, nv2, nv0);
-            step(I2{}, I1{}, mA, nA, dA_, mB, nB, dB_, true);
-            sync_step(I3{}, nv3, nv1);
-            step(I3{}, I2{}, mB, nB, dB_, mA, nA, dA_, true);
+            sync_step(I0{}, nv0);
+            step(I0{}, I3{}, mA, nA, dA_, mB, nB, dB_, k > 0, nv2);
+            sync_step(I1{}, nv1);
+            step(I1{}, I0{}, mB, nB, dB_, mA, nA, dA_, true, nv3);
+            sync_step(I2{}, nv2);
+            step(I2{}, I1{}, mA, nA, dA_, mB, nB, dB_, true, nv0);
+            sync_step(I3{}, nv3);
+            step(I3{}, I2{}, mB, nB, dB_, mA, nA, dA_, true, nv1);
         }
         if (k <= nt) {
-            sync_step(I0{}, nv0, nv2);
-            step(I0{}, I3{}, mA, nA, dA_, mB, nB, dB_, k > 0);
+            sync_step(I0{}, nv0);
+            step(I0{}, I3{}, mA, nA, dA_, mB, nB, dB_, k > 0, nv2);
             if (k + 1 <= nt) {
-                sync_step(I1{}, nv1, nv3);
-                step(I1{}, I0{}, mB, nB, dB_, mA, nA, dA_, true);
+                sync_step(I1{}, nv1);
+                step(I1{}, I0{}, mB, nB, dB_, mA, nA, dA_, true, nv3);
                 if (k + 2 <= nt) {
-                    sync_step(I2{}, nv2, nv0);
-                    step(I2{}, I1{}, mA, nA, dA_, mB, nB, dB_, true);
+                    sync_step(I2{}, nv2);
+                    step(I2{}, I1{}, mA, nA, dA_, mB, nB, dB_, true, nv0);
                 }
             }
         }

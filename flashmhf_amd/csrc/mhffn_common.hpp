@@ -240,8 +240,20 @@ __device__ __forceinline__ u32x4 lds_read16_async(unsigned addr)
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(IMM));
     return v;
 }
+// Two 4-byte values per lane, 128 bytes apart (one instruction, one LDS operation).
+__device__ __forceinline__ u32x2 lds_read2x4_async(unsigned addr)
+{
+    u32x2 v;
+    asm volatile("ds_read2_b32 %0, %1 offset1:32" : "=v"(v) : "v"(addr));
+    return v;
+}
 // At most N LDS operations of this wave still outstanding; the operands cannot be used above it.  Same conditions as
 // lds_tr_wait_n.
+template <int N>
+__device__ __forceinline__ void lds_wait_n(u32x4& a, u32x4& b, u32x2& c)
+{
+    asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(a), "+v"(b), "+v"(c) : "n"(N));
+}
 template <int N>
 __device__ __forceinline__ void lds_wait_n(u32x4& a, u32x4& b)
 {

@@ -43,6 +43,16 @@ constexpr int FWD_REGION_B = FWD_NST * TILE_B;   // 32 KB
 constexpr int FWD_V0 = 0, FWD_K0 = FWD_REGION_B, FWD_U0 = 2 * FWD_REGION_B;
 constexpr int FWD_RING_B = 3 * FWD_REGION_B;     // 96 KB
 
+// LDS operations issued behind the K/U reads of k-step ks up to the wait in front of that k-step's matrix instructions,
+// for the issue order of the block step (K/U of k-steps 0 and 1 up front; in k-step j first the four V^T reads of row
+// tile j - 1 while 1 <= j <= CT, then the two K/U reads of k-step j + 2).
+__host__ __device__ constexpr int fwd_younger_reads(int ks, int KS, int CT)
+{
+    int n = ks == 0 ? 2 : 0;                       // k-step 1's reads follow k-step 0's up front
+    for (int j = ks < 2 ? 0 : ks - 1; j <= ks; ++j) n += (j >= 1 && j <= CT ? 4 : 0) + (j + 2 < KS ? 2 : 0);
+    return n;
+}
+
 template <int DH>
 __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
 {
@@ -120,14 +130,12 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
 
     const int krow = row_perm32(l32);
     const TrLane<CT> trl = make_tr_lane<CT, 8, 4>(lane);
-    // per-lane bases of the K and U row reads for every k-step (stage 0); the stage is added as an immediate
-    const unsigned char* kbase[KS];
-    const unsigned char* ubase[KS];
+    // per-lane LDS addresses of the K row reads for every k-step (stage 0); the stage, and the distance to the U region,
+    // go into the instruction's immediate offset
+    unsigned kaddr[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        kbase[ks] = smem + FWD_K0 + krow * TILE_ROW_B + (((2 * ks + g) ^ swz16(krow)) << 4);
-        ubase[ks] = kbase[ks] + (FWD_U0 - FWD_K0);
-    }
+    for (int ks = 0; ks < KS; ++ks)
+        kaddr[ks] = lds_addr(smem) + FWD_K0 + krow * TILE_ROW_B + (((2 * ks + g) ^ swz16(krow)) << 4);
     const unsigned smem0 = lds_addr(smem);
 
     // consumes M/N of block blk (mc, nc), produces M/N of block blk+1 (mn, nn); ST = blk % FWD_NST
@@ -135,35 +143,33 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
         constexpr int ST = decltype(st_)::value, STN = (ST + 1) % FWD_NST;
         wait_vmcnt<FILL>();   // blocks <= blk+1 have landed (only block blk+2's loads may be in flight)
         __syncthreads();      // ... for every wave; and every wave is done with the stage about to be refilled
-        issue_block(blk + 3, (ST + 3) % FWD_NST);
 
-        // The gate value enters through its reciprocal: r / (1 + e) = 1 / fma(e, 1/r, 1/r), one multiply fewer per
-        // element.  1/r is clamped to the largest finite float, so a zero gate makes the denominator at least FLT_MAX, whose
-        // reciprocal the hardware flushes to exactly 0.
-        float rinv[2];
-#pragma unroll
-        for (int ct = 0; ct < 2; ++ct) {
-            const float rv = sR[(e & (GATE_WIN - 1)) * BT + wave * 64 + ct * 32 + l32];
-            rinv[ct] = __builtin_amdgcn_fmed3f(__builtin_amdgcn_rcpf(rv), -FLT_MAX_F, FLT_MAX_F);
-        }
-        auto read_k = [&](int ks) { return *reinterpret_cast<const bf16x8*>(kbase[ks] + STN * TILE_B); };
-        auto read_u = [&](int ks) { return *reinterpret_cast<const bf16x8*>(ubase[ks] + STN * TILE_B); };
-
-        // V^T operands of this block's second product first: these reads are issued from inline assembly, so the
-        // compiler's own lgkmcnt bookkeeping for the K/U reads below does not know them; LDS returns in order, so any of
-        // its waits that followed them would silently wait for them too.  Issued ahead of every other LDS read of the
-        // step they never delay a wait.
+        // LDS reads of the step, all issued from inline assembly and waited for by count (the compiler's own waits are
+        // full ones: behind a group of reads in flight it waits for the youngest along with the one it needs).  Issue
+        // order: the two gate values, the K/U operands of k-steps 0 and 1, then per k-step ks the V^T operands of row tile
+        // ks - 1 (for the second product, long after) and the K/U operands of k-step ks + 2.  LDS operations complete in
+        // order, so "at most younger(ks) outstanding" means the operands of k-step ks have arrived; the last k-step's
+        // wait is a full one and covers the V^T operands.
+        u32x2 rvu = lds_read2x4_async(lds_addr(sR + (e & (GATE_WIN - 1)) * BT + wave * 64 + l32));
         TrOperand av[CT][2];
-#pragma unroll
-        for (int i = 0; i < CT; ++i) {
+        u32x4 ak[3], au[3];   // K/U operand ring, two k-steps ahead
+        auto request = [&](auto kc) {
+            constexpr int ks = decltype(kc)::value;
+            ak[ks % 3] = lds_read16_async<STN * TILE_B>(kaddr[ks]);
+            au[ks % 3] = lds_read16_async<FWD_U0 - FWD_K0 + STN * TILE_B>(kaddr[ks]);
+        };
+        auto request_v = [&](auto ic) {
+            constexpr int i = decltype(ic)::value;
             av[i][0] = tile_read_cols_async<FWD_V0 + ST * TILE_B>(smem0, trl, i);
             av[i][1] = tile_read_cols_async<FWD_V0 + ST * TILE_B + 4096>(smem0, trl, i);
-        }
-        bf16x8 ak[3], au[3];   // K/U operand ring, two k-steps ahead
-        ak[0] = read_k(0);
-        au[0] = read_u(0);
-        ak[1] = read_k(1);
-        au[1] = read_u(1);
+        };
+        request(std::integral_constant<int, 0>{});
+        request(std::integral_constant<int, 1>{});
+        // the fill of the stage that has just come free is issued behind the first reads: its address arithmetic and six
+        // instructions pass while those reads are on their way
+        __builtin_amdgcn_sched_barrier(0);
+        issue_block(blk + 3, (ST + 3) % FWD_NST);
+        float rinv[2];
         bf16x8 pt[2][2];
         float e0 = 0, e1 = 0, xn0 = 0, xn1 = 0;   // carried between the chunks of one element pair
         __builtin_amdgcn_sched_barrier(0);
@@ -192,16 +198,30 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
             constexpr int k = decltype(k_)::value;
             if constexpr (k < NG1) {
                 constexpr int ks = k / 4, w = k % 4, ct = w >> 1;
-                if constexpr (w == 0 && ks + 2 < KS) {
-                    ak[(ks + 2) % 3] = read_k(ks + 2);
-                    au[(ks + 2) % 3] = read_u(ks + 2);
+                if constexpr (w == 0) {
+                    if constexpr (ks >= 1 && ks <= CT) request_v(std::integral_constant<int, ks - 1>{});
+                    if constexpr (ks + 2 < KS) request(std::integral_constant<int, ks + 2>{});
+                    if constexpr (ks == 0) {
+                        lds_wait_n<fwd_younger_reads(0, KS, CT)>(ak[0], au[0], rvu);     // (the gate values are older)
+                        // The gate value enters through its reciprocal: r / (1 + e) = 1 / fma(e, 1/r, 1/r), one multiply
+                        // fewer per element.  1/r is clamped to the largest finite float, so a zero gate makes the
+                        // denominator at least FLT_MAX, whose reciprocal the hardware flushes to exactly 0.
+#pragma unroll
+                        for (int c2 = 0; c2 < 2; ++c2) {
+                            const unsigned bits = rvu[c2];    // (a scalar copy: the cast below must not see a vector element)
+                            rinv[c2] = __builtin_amdgcn_fmed3f(__builtin_amdgcn_rcpf(__builtin_bit_cast(float, bits)),
+                                                               -FLT_MAX_F, FLT_MAX_F);
+                        }
+                    } else {
+                        lds_wait_n<fwd_younger_reads(ks, KS, CT)>(ak[ks % 3], au[ks % 3]);
+                    }
                 }
                 if constexpr ((w & 1) == 0) {
-                    if constexpr (ks == 0) mfma32_vgpr_first_bacc(mn[ct], ak[0], q[ct][0]);
-                    else mfma32_vgpr_acc_bacc(mn[ct], ak[ks % 3], q[ct][ks]);
+                    if constexpr (ks == 0) mfma32_vgpr_first_bacc(mn[ct], __builtin_bit_cast(bf16x8, ak[0]), q[ct][0]);
+                    else mfma32_vgpr_acc_bacc(mn[ct], __builtin_bit_cast(bf16x8, ak[ks % 3]), q[ct][ks]);
                 } else {
-                    if constexpr (ks == 0) mfma32_vgpr_first_bacc(nn[ct], au[0], q[ct][0]);
-                    else mfma32_vgpr_acc_bacc(nn[ct], au[ks % 3], q[ct][ks]);
+                    if constexpr (ks == 0) mfma32_vgpr_first_bacc(nn[ct], __builtin_bit_cast(bf16x8, au[0]), q[ct][0]);
+                    else mfma32_vgpr_acc_bacc(nn[ct], __builtin_bit_cast(bf16x8, au[ks % 3]), q[ct][ks]);
                 }
             } else {
                 constexpr int g2 = k - NG1, s = g2 / (2 * CT), ct = (g2 / CT) % 2, i = g2 % CT;
@@ -230,7 +250,7 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
     {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const bf16x8 a = *reinterpret_cast<const bf16x8*>(kbase[ks]), u = *reinterpret_cast<const bf16x8*>(ubase[ks]);
+            const bf16x8 a = tile_read_rows(smem + FWD_K0, krow, ks, g), u = tile_read_rows(smem + FWD_U0, krow, ks, g);
 #pragma unroll
             for (int ct = 0; ct < 2; ++ct) {
                 if (ks == 0) { mfma32_vgpr_first_bacc(mA[ct], a, q[ct][0]); mfma32_vgpr_first_bacc(nA[ct], u, q[ct][0]); }
