@@ -148,8 +148,8 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
         // full ones: behind a group of reads in flight it waits for the youngest along with the one it needs).  Issue
         // order: the two gate values, the K/U operands of k-steps 0 and 1, then per k-step ks the V^T operands of row tile
         // ks - 1 (for the second product, long after) and the K/U operands of k-step ks + 2.  LDS operations complete in
-        // order, so "at most younger(ks) outstanding" means the operands of k-step ks have arrived; the last k-step's
-        // wait is a full one and covers the V^T operands.
+        // order, so "at most younger(ks) outstanding" means the operands of k-step ks have arrived; the V^T operands
+        // have a full wait of their own in front of the second product, by when they have long landed.
         u32x2 rvu = lds_read2x4_async(lds_addr(sR + (e & (GATE_WIN - 1)) * BT + wave * 64 + l32));
         TrOperand av[CT][2];
         u32x4 ak[3], au[3];   // K/U operand ring, two k-steps ahead
