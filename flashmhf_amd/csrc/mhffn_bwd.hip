@@ -6,6 +6,8 @@
 //          dR_e += sum_j dA * silu(M) * N                      (fp32, before any rounding)
 //          dN^T = r_e dA^T silu(M^T),  dM^T = r_e dA^T N^T silu'(M^T)      (rounded once to bf16)
 //          dQ^T += K^T dM^T + U^T dN^T                         (K^T, U^T: transposing reads of the same K, U tiles)
+//      The two waves of a SIMD work half a block apart (one's element-wise phase under the other's matrix phases),
+//      the later one at a higher wave priority.
 //      Formulas: kernels/triton/flash_mlp_moe.py:401-414, :527-542.
 //
 //  (2) dK/dU/dV kernel -- a wave owns one 32-row block of K/U/V (held in registers as MFMA B operands) and loops
@@ -42,7 +44,7 @@ __global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
     constexpr int BT = NW * 32;
     constexpr int FILL = 24 / NW;          // tile-fill wave-instructions per wave and block (3 tiles x 8 / NW waves)
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-    float* sR = reinterpret_cast<float*>(smem + DQ_NST * DQ_STAGE_B);   // [min(E, GATE_WIN)][BT]: one expert window
+    float* sR = reinterpret_cast<float*>(smem + DQ_NST * DQ_STAGE_B);   // [min(E, 64)][BT]: expert e in slot e % 64
 
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -82,21 +84,21 @@ __global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
     }
     issue_block(0);
     // Gate values of the workgroup's 256 tokens, expert-major [E][BT]: asynchronous 4-byte LDS-direct loads, lane = token;
-    // a pair of waves shares a group of 64 tokens and takes the even and the odd experts.  LDS holds a window of GATE_WIN
-    // experts at a time; the first is issued between block 0 and block 1, so that the first wait for block 0 covers it
-    // too, and a layer with more experts restages the tile at the top of the expert loop.
+    // a pair of waves shares a group of 64 tokens and takes the even and the odd experts.  LDS holds 64 experts, expert e
+    // in slot e % 64; the first 64 are issued between block 0 and block 1, so that the first wait for block 0 covers
+    // them too, and a layer with more experts refills the slots 32 at a time as the block loop leaves them behind.
     const float* rrow;
     {
         int t = tb * BT + (wave >> 1) * 64 + lane;
         t = t < p.S ? t : p.S - 1;
         rrow = p.R + (rowbase + t) * p.E;
     }
-    auto stage_gates = [&](int e0) {
-        const int e1 = e0 + GATE_WIN < p.E ? e0 + GATE_WIN : p.E;
+    auto stage_gates = [&](int e0, int e1) {
+        e1 = e1 < p.E ? e1 : p.E;
         for (int e = e0 + (wave & 1); e < e1; e += 2)
-            __builtin_amdgcn_global_load_lds((gptr_t)(rrow + e), (lptr_t)(sR + (e - e0) * BT + (wave >> 1) * 64), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(rrow + e), (lptr_t)(sR + (e & 63) * BT + (wave >> 1) * 64), 4, 0, 0);
     };
-    stage_gates(0);
+    stage_gates(0, 64);
     issue_block(1);
 
     f32x16 dq[CT];
@@ -107,101 +109,135 @@ __global__ __launch_bounds__(512) void mhffn_bwd_dqdr_kernel(DqArgs p)
 
     const int krow = row_perm32(l32);
     const TrLane<CT> trl = make_tr_lane<CT, 8, 4>(lane);
-    int blk = 0;
-    for (int e = 0; e < p.E; ++e) {
-        if (e > 0 && (e & (GATE_WIN - 1)) == 0) {
-            __syncthreads();      // every wave has read its gate values of the window before
-            stage_gates(e);
-            wait_vmcnt<0>();      // (also lands the blocks in flight; the next wait for a block then passes at once)
-            __syncthreads();
+    // One block takes three phases per wave: first products (24 matrix instructions for d_h = 128), element-wise work
+    // (VALU only), second products (16 matrix instructions).  The two waves that share a SIMD run them in opposite phase
+    // between two barriers -- waves 0..3: first(b), element-wise(b), second(b); waves 4..7: element-wise(b-1),
+    // second(b-1), first(b) -- so that one wave's VALU phase lies under the other's matrix phases.  Left to the
+    // hardware's oldest-first arbitration the early waves win every conflict and then idle at the barrier while the late
+    // waves catch up alone; the late waves therefore run at a higher wave priority, which evens the two out.  The late
+    // waves carry M, N, dA of block b across the barrier and need one more trip at the end; the ring keeps block b-1
+    // alive that long (the refill behind barrier b targets the stage of block b-2).
+    f32x16 m, n, da;
+    bf16x8 dmt[2], dnt[2];
+    float dr = 0.0f;
+    auto first_products = [&](int blk) {
+        const unsigned char* sK = smem + (blk % DQ_NST) * DQ_STAGE_B;
+        const unsigned char* sU = sK + TILE_B;
+        const unsigned char* sV = sU + TILE_B;
+#pragma unroll
+        for (int x = 0; x < 16; ++x) { m[x] = 0.0f; n[x] = 0.0f; da[x] = 0.0f; }
+        // The K/U/V operands come from LDS through a ring of three register sets, read two k-steps ahead of the
+        // matrix instructions that use them; the fence after each k-step keeps the compiler from gathering the
+        // reads back to the front (which costs their whole latency once per block).
+        bf16x8 ak[3], au[3], av[3];
+#pragma unroll
+        for (int k0 = 0; k0 < 2; ++k0) {
+            ak[k0] = tile_read_rows(sK, krow, k0, g);
+            au[k0] = tile_read_rows(sU, krow, k0, g);
+            av[k0] = tile_read_rows(sV, krow, k0, g);
         }
-        float dr = 0.0f;
-        for (int jb = 0; jb < p.nbe; ++jb, ++blk) {
-            wait_vmcnt<FILL>();       // block blk has landed (block blk+1 may be in flight)
-            __syncthreads();
-            issue_block(blk + 2);
-
-            const unsigned char* sK = smem + (blk % DQ_NST) * DQ_STAGE_B;
-            const unsigned char* sU = sK + TILE_B;
-            const unsigned char* sV = sU + TILE_B;
-            const float r = sR[(e & (GATE_WIN - 1)) * BT + wave * 32 + l32];
-
-            f32x16 m, n, da;
-#pragma unroll
-            for (int x = 0; x < 16; ++x) { m[x] = 0.0f; n[x] = 0.0f; da[x] = 0.0f; }
-            {
-                // The K/U/V operands come from LDS through a ring of three register sets, read two k-steps ahead of the
-                // matrix instructions that use them; the fence after each k-step keeps the compiler from gathering the
-                // reads back to the front (which costs their whole latency once per block).
-                bf16x8 ak[3], au[3], av[3];
-#pragma unroll
-                for (int k0 = 0; k0 < 2; ++k0) {
-                    ak[k0] = tile_read_rows(sK, krow, k0, g);
-                    au[k0] = tile_read_rows(sU, krow, k0, g);
-                    av[k0] = tile_read_rows(sV, krow, k0, g);
-                }
-                static_for<KS>([&](auto kc) {
-                    constexpr int ks = decltype(kc)::value;
-                    if constexpr (ks + 2 < KS) {
-                        ak[(ks + 2) % 3] = tile_read_rows(sK, krow, ks + 2, g);
-                        au[(ks + 2) % 3] = tile_read_rows(sU, krow, ks + 2, g);
-                        av[(ks + 2) % 3] = tile_read_rows(sV, krow, ks + 2, g);
-                    }
-                    m = mfma32(ak[ks % 3], q[ks], m);
-                    n = mfma32(au[ks % 3], q[ks], n);
-                    da = mfma32(av[ks % 3], go[ks], da);
-                    __builtin_amdgcn_sched_barrier(0);
-                });
+        static_for<KS>([&](auto kc) {
+            constexpr int ks = decltype(kc)::value;
+            if constexpr (ks + 2 < KS) {
+                ak[(ks + 2) % 3] = tile_read_rows(sK, krow, ks + 2, g);
+                au[(ks + 2) % 3] = tile_read_rows(sU, krow, ks + 2, g);
+                av[(ks + 2) % 3] = tile_read_rows(sV, krow, ks + 2, g);
             }
-
-            bf16x8 dmt[2], dnt[2];
-#pragma unroll
-            for (int s = 0; s < 2; ++s)
-#pragma unroll
-                for (int kk = 0; kk < 8; ++kk) {
-                    const int i = 8 * s + kk;
-                    const float x = m[i], nn = n[i], a = da[i];
-                    const float sg = fast_sigmoid(x);
-                    const float sl = x * sg;                 // silu(m)
-                    const float as = a * sl;
-                    dr = __builtin_fmaf(as, nn, dr);
-                    const float w = __builtin_fmaf(sl, 1.0f - sg, sg);    // silu'(m)
-                    dnt[s][kk] = (bf16_t)(r * as);
-                    dmt[s][kk] = (bf16_t)((r * a) * (nn * w));
-                }
-
-            // second products: operand pairs (Kt, Ut) are requested two steps ahead of the MFMAs that consume them; the
-            // region is fenced so that the partial LDS waits below count exactly these reads
+            m = mfma32(ak[ks % 3], q[ks], m);
+            n = mfma32(au[ks % 3], q[ks], n);
+            da = mfma32(av[ks % 3], go[ks], da);
             __builtin_amdgcn_sched_barrier(0);
-            {
-                constexpr int NSET = 2 * CT;          // (s, i) in s-major order
-                TrOperand tk[3], tu[3];
-                auto request = [&](auto ic) {
-                    constexpr int idx = decltype(ic)::value;
-                    constexpr int s = idx / CT, i = idx % CT;
-                    tk[idx % 3] = tile_read_cols_async<4096 * s>(lds_addr(sK), trl, i);
-                    tu[idx % 3] = tile_read_cols_async<4096 * s + TILE_B>(lds_addr(sK), trl, i);
-                };
-                request(std::integral_constant<int, 0>{});
-                request(std::integral_constant<int, 1>{});
-                static_for<NSET>([&](auto ic) {
-                    constexpr int idx = decltype(ic)::value;
-                    constexpr int s = idx / CT, i = idx % CT;
-                    if constexpr (idx + 2 < NSET) request(std::integral_constant<int, idx + 2>{});
-                    constexpr int ahead = (NSET - 1 - idx) < 2 ? (NSET - 1 - idx) : 2;
-                    lds_tr_wait_n<4 * ahead>(tk[idx % 3], tu[idx % 3]);
-                    dq[i] = mfma32(tr_value(tk[idx % 3]), dmt[s], dq[i]);
-                    dq[i] = mfma32(tr_value(tu[idx % 3]), dnt[s], dq[i]);
-                });
+        });
+    };
+    auto element_wise = [&](float r) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                const int i = 8 * s + kk;
+                const float x = m[i], nn = n[i], a = da[i];
+                const float sg = fast_sigmoid(x);
+                const float sl = x * sg;                 // silu(m)
+                const float as = a * sl;
+                dr = __builtin_fmaf(as, nn, dr);
+                const float w = __builtin_fmaf(sl, 1.0f - sg, sg);    // silu'(m)
+                dnt[s][kk] = (bf16_t)(r * as);
+                dmt[s][kk] = (bf16_t)((r * a) * (nn * w));
             }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // dR[t, e]: the two lane halves hold disjoint j rows of the same token column.
+    };
+    // second products: operand pairs (Kt, Ut) are requested two steps ahead of the MFMAs that consume them; the region is
+    // fenced so that the partial LDS waits count exactly these reads
+    auto second_products = [&](int blk) {
+        const unsigned sK = lds_addr(smem + (blk % DQ_NST) * DQ_STAGE_B);
+        __builtin_amdgcn_sched_barrier(0);
         {
+            constexpr int NSET = 2 * CT;          // (s, i) in s-major order
+            TrOperand tk[3], tu[3];
+            auto request = [&](auto ic) {
+                constexpr int idx = decltype(ic)::value;
+                constexpr int s = idx / CT, i = idx % CT;
+                tk[idx % 3] = tile_read_cols_async<4096 * s>(sK, trl, i);
+                tu[idx % 3] = tile_read_cols_async<4096 * s + TILE_B>(sK, trl, i);
+            };
+            request(std::integral_constant<int, 0>{});
+            request(std::integral_constant<int, 1>{});
+            static_for<NSET>([&](auto ic) {
+                constexpr int idx = decltype(ic)::value;
+                constexpr int s = idx / CT, i = idx % CT;
+                if constexpr (idx + 2 < NSET) request(std::integral_constant<int, idx + 2>{});
+                constexpr int ahead = (NSET - 1 - idx) < 2 ? (NSET - 1 - idx) : 2;
+                lds_tr_wait_n<4 * ahead>(tk[idx % 3], tu[idx % 3]);
+                dq[i] = mfma32(tr_value(tk[idx % 3]), dmt[s], dq[i]);
+                dq[i] = mfma32(tr_value(tu[idx % 3]), dnt[s], dq[i]);
+            });
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    int e = 0, jb = 0;          // expert and block-in-expert of the block whose element-wise work comes next
+    auto finish_block = [&](int blk) {
+        element_wise(sR[(e & 63) * BT + wave * 32 + l32]);
+        second_products(blk);
+        if (++jb == p.nbe) {
+            // dR[t, e]: the two lane halves hold disjoint j rows of the same token column.
             const float tot = dr + __shfl_xor(dr, 32);
             const int t = tok0 + l32;
             if (g == 0 && t < p.S) p.dR[(rowbase + t) * p.E + e] = tot;
+            dr = 0.0f;
+            jb = 0;
+            ++e;
+            // More than 64 experts: with expert 32k behind it (k >= 1), this pair of waves refills the slots of experts
+            // 32k-32 .. 32k-1 with experts 32k+32 .. 32k+63 of its own 64 tokens.  Its partner is in the same interval
+            // between two barriers, so at a block of expert 32k or later; the values are first read 31 experts on, and
+            // every barrier's wait on the way leaves at most three of this wave's loads outstanding.
+            if (e > 1 && (e & 31) == 1 && e + 31 < p.E) stage_gates(e + 31, e + 63);
         }
+    };
+    // Barrier b: block b has landed for every wave, and every wave is done with block b - 2, whose stage the fill of
+    // block b + 2 takes.
+    auto next_interval = [&](int b) {
+        wait_vmcnt<FILL>();       // block b has landed (block b+1 may be in flight)
+        __syncthreads();
+        issue_block(b + 2);
+    };
+    if (wave < NW / 2) {
+        for (int b = 0; b < nblk; ++b) {
+            next_interval(b);
+            first_products(b);
+            finish_block(b);
+        }
+        next_interval(nblk);      // the barrier of the late waves' extra trip
+    } else {
+        __builtin_amdgcn_s_setprio(2);
+        next_interval(0);
+        first_products(0);
+        for (int b = 1; b < nblk; ++b) {
+            next_interval(b);
+            finish_block(b - 1);
+            first_products(b);
+        }
+        next_interval(nblk);
+        finish_block(nblk - 1);
+        __builtin_amdgcn_s_setprio(0);
     }
     wait_vmcnt<0>();   // drain the phantom prefetches: they write the ring, which the epilogue reuses
     __syncthreads();   // every wave is done reading the ring
