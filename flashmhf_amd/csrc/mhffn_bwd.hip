@@ -571,7 +571,7 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
 #pragma unroll
                 for (int a = 0; a < 4; ++a) rv[a] = __builtin_bit_cast(f32x4, rvu[a]);
             } else {
-                lds_wait_n<younger>(aq[ks % 3], ag[ks % 3]);
+                lds_wait_n<younger>();        // (consumed by asm matrix instructions only)
             }
             const bf16x8 aqv = __builtin_bit_cast(bf16x8, aq[ks % 3]), agv = __builtin_bit_cast(bf16x8, ag[ks % 3]);
             if constexpr (ks == 0) mfma32_vgpr_first_bacc(m, aqv, kB[0]);

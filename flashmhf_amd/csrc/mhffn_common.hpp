@@ -254,6 +254,14 @@ __device__ __forceinline__ void lds_wait_n(u32x4& a, u32x4& b, u32x2& c)
 {
     asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(a), "+v"(b), "+v"(c) : "n"(N));
 }
+// The same without operands, for reads whose only consumers are matrix instructions issued from inline assembly (volatile
+// statements keep their order): with the operands tied to the wait the compiler assumes the statement wrote them and puts
+// a hazard s_nop in front of the matrix instruction.
+template <int N>
+__device__ __forceinline__ void lds_wait_n()
+{
+    asm volatile("s_waitcnt lgkmcnt(%0)" :: "n"(N));
+}
 template <int N>
 __device__ __forceinline__ void lds_wait_n(u32x4& a, u32x4& b)
 {

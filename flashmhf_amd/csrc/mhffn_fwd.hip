@@ -213,7 +213,7 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
                                                                -FLT_MAX_F, FLT_MAX_F);
                         }
                     } else {
-                        lds_wait_n<fwd_younger_reads(ks, KS, CT)>(ak[ks % 3], au[ks % 3]);
+                        lds_wait_n<fwd_younger_reads(ks, KS, CT)>();     // (consumed by asm matrix instructions only)
                     }
                 }
                 if constexpr ((w & 1) == 0) {
