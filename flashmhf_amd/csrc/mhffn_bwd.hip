@@ -454,9 +454,19 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
     // this address ^ (ks << 5): the ring starts on a 1 KB boundary, so the exclusive-or commutes with the sum
     const unsigned qaddr = lds_addr(smem_raw) + l32 * 256 + ((g ^ fr) << 4);
 
+    // B operands of the token contraction (P, dM, dN of one tile, bf16).  They live across steps: the element pairs 0 and 1
+    // of a tile are converted under the last matrix instructions of the step that computed its first products, the other
+    // six under the next step's first 36.  Zero for the tile that does not exist before the first one.
+    bf16x8 pB[2], dmB[2], dnB[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) { pB[s][kk] = (bf16_t)0.0f; dmB[s][kk] = (bf16_t)0.0f; dnB[s][kk] = (bf16_t)0.0f; }
+
     // first products of the tile in stage ST -> (m, n, da) in architectural VGPRs, element-wise work of the PREVIOUS
-    // tile (registers pm, pn, pda; gate values from stage SP) dealt out between the k-steps so that the VALU works
-    // under the MFMAs; then the token contraction of the previous tile.
+    // tile (registers pm, pn, pda; gate values from stage SP) dealt out between the matrix instructions so that the VALU
+    // works under them; then the token contraction of the previous tile, with the first element pairs of THIS tile's
+    // element-wise work under its last matrix instructions.
     //   registers 4a+b of m/n/da: token 8a + 4g + b (rows), column j = l32.
     auto step = [&](auto st_c, auto sp_c, f32x16& m, f32x16& n, f32x16& da, const f32x16& pm, const f32x16& pn,
                     const f32x16& pda, bool live, int& nv_next) {
@@ -469,11 +479,12 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         // phantom steps that pad the loop): a zero gate makes P, dM and dN exactly zero
         const float* pR = live ? reinterpret_cast<const float*>(pG + TILE_B) + wave * 64 : sZero;
 
-        bf16x8 pB[2], dmB[2], dnB[2];
-        // LDS reads of the first products: the gate values of the previous tile for this lane's 16 token rows (4
+        // LDS reads of the first products: the gate values of this tile's first four token rows (for the element pairs
+        // converted at the end of this step) and of the previous tile for this lane's 16 token rows (4
         // consecutive rows per 16-byte read), then the operand ring (k-step ks + 2 is requested while ks is consumed).
         // All are issued from inline assembly and waited for by count; the element-wise slices in between are VALU only.
         __builtin_amdgcn_sched_barrier(0);
+        u32x4 rvn = lds_read16_async<0>(lds_addr(smem_raw) + (ST * DW_STAGE_B + 2 * TILE_B) + wave * 256 + 16 * g);
         u32x4 rvu[4];
         {
             const unsigned ra = lds_addr(pR) + 16 * g;
@@ -514,51 +525,58 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
         // fits under one MFMA (32 cycles).  With sigma = 1/(1+2^(-m log2 e)), B = r sigma, A = m B (= r silu(m)):
         //     P = A n,   dN = A dA,   dM = (B + A (1 - sigma)) (n dA)         [silu'(m) = sigma + silu(m) (1 - sigma)]
         float ex[8][2], sg[8][2], nda[8][2], Av[8][2], Bv[8][2], s1[8][2];
-        auto slice = [&](auto pc, auto kc) {
+        f32x4 rvn4;                                   // gate values of THIS tile's token rows 4g .. 4g+3 (elements 0..3)
+        auto slice_on = [&](auto pc, auto kc, const f32x16& sm, const f32x16& sn, const f32x16& sda, auto gate) {
             constexpr int pr = decltype(pc)::value, k = decltype(kc)::value;
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const int i = 2 * pr + u;
                 if constexpr (k == 0) {
-                    ex[pr][u] = __builtin_amdgcn_exp2f(-LOG2E * pm[i]);
+                    ex[pr][u] = __builtin_amdgcn_exp2f(-LOG2E * sm[i]);
                 } else if constexpr (k == 1) {
                     sg[pr][u] = __builtin_amdgcn_rcpf(1.0f + ex[pr][u]);
-                    nda[pr][u] = pn[i] * pda[i];
+                    nda[pr][u] = sn[i] * sda[i];
                 } else if constexpr (k == 2) {
-                    Bv[pr][u] = rv[i >> 2][i & 3] * sg[pr][u];
-                    Av[pr][u] = pm[i] * Bv[pr][u];
+                    Bv[pr][u] = gate(i) * sg[pr][u];
+                    Av[pr][u] = sm[i] * Bv[pr][u];
                     s1[pr][u] = 1.0f - sg[pr][u];
                 } else if constexpr (k == 3) {
-                    pB[i >> 3][i & 7] = (bf16_t)(Av[pr][u] * pn[i]);
-                    dnB[i >> 3][i & 7] = (bf16_t)(Av[pr][u] * pda[i]);
+                    pB[i >> 3][i & 7] = (bf16_t)(Av[pr][u] * sn[i]);
+                    dnB[i >> 3][i & 7] = (bf16_t)(Av[pr][u] * sda[i]);
                 } else {
                     dmB[i >> 3][i & 7] = (bf16_t)(__builtin_fmaf(Av[pr][u], s1[pr][u], Bv[pr][u]) * nda[pr][u]);
                 }
             }
         };
-        // Slice list 1 (24 entries, placed behind the first-product MFMAs): pairs 0..3 completely -- the s = 0 operands of
-        // the contraction -- then the exponentials of pairs 4..7.  Slice list 2 (16 entries, behind the s = 0 contraction
-        // MFMAs): the rest of pairs 4..7, which the s = 1 MFMAs need.
-        auto list1 = [&](auto qc) {
-            constexpr int q = decltype(qc)::value;
-            if constexpr (q < 20) slice(std::integral_constant<int, q / 5>{}, std::integral_constant<int, q % 5>{});
-            else slice(std::integral_constant<int, q - 16>{}, std::integral_constant<int, 0>{});
-        };
-        auto list2 = [&](auto qc) {
-            constexpr int q = decltype(qc)::value;
-            slice(std::integral_constant<int, 4 + q / 4>{}, std::integral_constant<int, 1 + q % 4>{});
-        };
-
-        // Phase 1: first products of this tile (24 MFMAs for d_h = 128), one slice of list 1 behind each: back-to-back
-        // MFMAs would block this wave's in-order instruction stream until the matrix pipe takes each.
-        constexpr int NS1 = 3 * KS;
-        auto after_slot1 = [&](auto kc) {
+        // The 40 slices of a tile (8 element pairs x 5) are spread over 48 consecutive matrix instructions for d_h = 128
+        // (NSL in general): pairs 0 and 1 of THIS tile behind the last 3 CT of this step (the s = 1 half of the
+        // contraction, which reads only the operand halves of elements 8..15), pairs 2..7 of the PREVIOUS tile behind
+        // this step's first NSL - 3 CT.  Pairs 2 and 3 are done long before the s = 0 half starts, pairs 4..7 before the
+        // s = 1 half.  Each matrix instruction so has about one slice behind it; two slices behind one cost the wave
+        // more issue time than the instruction's 32 cycles, none leaves the matrix pipe's shadow unused.
+        constexpr int NS1 = 3 * KS, NSL = NS1 + 6 * CT, NLATE = 3 * CT, NEARLY = NSL - NLATE;
+        static_assert(9 * NEARLY / 30 < NS1, "pairs 2 and 3 must be converted before the s = 0 half of the contraction");
+        auto ew_slot = [&](auto kc) {
             constexpr int k = decltype(kc)::value;
-            static_for<24>([&](auto qc) {
-                if constexpr (decltype(qc)::value * NS1 / 24 == k) list1(qc);
-            });
+            if constexpr (k < NEARLY) {
+                static_for<30>([&](auto qc) {
+                    constexpr int q = decltype(qc)::value;
+                    if constexpr (q * NEARLY / 30 == k)
+                        slice_on(std::integral_constant<int, 2 + q / 5>{}, std::integral_constant<int, q % 5>{}, pm, pn, pda,
+                                 [&](int i) { return rv[i >> 2][i & 3]; });
+                });
+            } else {
+                static_for<10>([&](auto qc) {
+                    constexpr int q = decltype(qc)::value;
+                    if constexpr (NEARLY + q * NLATE / 10 == k)
+                        slice_on(std::integral_constant<int, q / 5>{}, std::integral_constant<int, q % 5>{}, m, n, da,
+                                 [&](int i) { return rvn4[i & 3]; });
+                });
+            }
             __builtin_amdgcn_sched_barrier(0);
         };
+        auto after_slot1 = [&](auto kc) { ew_slot(kc); };
+
         static_for<KS>([&](auto kc) {
             constexpr int ks = decltype(kc)::value;
             if constexpr (ks + 2 < KS) request(std::integral_constant<int, ks + 2>{});
@@ -570,6 +588,8 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
                 lds_wait_n<younger>(aq[0], ag[0], rvu[0], rvu[1], rvu[2], rvu[3]);       // (the gate values are older)
 #pragma unroll
                 for (int a = 0; a < 4; ++a) rv[a] = __builtin_bit_cast(f32x4, rvu[a]);
+                asm volatile("" : "+v"(rvn));     // (older than the reads just waited for; no use of it may move above)
+                rvn4 = __builtin_bit_cast(f32x4, rvn);
             } else {
                 lds_wait_n<younger>();        // (consumed by asm matrix instructions only)
             }
@@ -598,23 +618,17 @@ __global__ __launch_bounds__(256) void mhffn_bwd_dkdudv_kernel(DwArgs p)
                 if constexpr (idx + 2 < NSET) request_tr(std::integral_constant<int, idx + 2>{});
                 constexpr int ahead = (NSET - 1 - idx) < 2 ? (NSET - 1 - idx) : 2;
                 lds_tr_wait_n<4 * ahead>(tq[idx % 3], tg[idx % 3]);
-                // s = 0: list 2 is dealt out over the 3 CT MFMAs of this half
+                // (element-wise slices behind each matrix instruction: see ew_slot)
                 auto after_slot2 = [&](auto kc) {
-                    constexpr int k = decltype(kc)::value;
-                    if constexpr (s == 0) {
-                        static_for<16>([&](auto qc) {
-                            if constexpr (decltype(qc)::value * (3 * CT) / 16 == k) list2(qc);
-                        });
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
+                    ew_slot(std::integral_constant<int, NS1 + 3 * idx + decltype(kc)::value>{});
                 };
                 dk[ct] = mfma32(tr_value(tq[idx % 3]), dmB[s], dk[ct]);
                 if constexpr (idx == NSET - 1 && !TAIL) prepare_tile();     // scalar work of the next fill, under this MFMA
-                after_slot2(std::integral_constant<int, 3 * ct>{});
+                after_slot2(std::integral_constant<int, 0>{});
                 du[ct] = mfma32(tr_value(tq[idx % 3]), dnB[s], du[ct]);
-                after_slot2(std::integral_constant<int, 3 * ct + 1>{});
+                after_slot2(std::integral_constant<int, 1>{});
                 dv[ct] = mfma32(tr_value(tg[idx % 3]), pB[s], dv[ct]);
-                after_slot2(std::integral_constant<int, 3 * ct + 2>{});
+                after_slot2(std::integral_constant<int, 2>{});
             });
         }
         __builtin_amdgcn_sched_barrier(0);

@@ -175,22 +175,27 @@ __global__ __launch_bounds__(256) void mhffn_fwd_kernel(FwdArgs p)
         __builtin_amdgcn_sched_barrier(0);
 
         // chunk c: third c%3 of element pair c/3; pairs ordered (tile 0, s 0), (tile 1, s 0), (tile 0, s 1), (tile 1, s 1)
-        // so that each second-product operand P^T[ct][s] is complete well before the slot that consumes it
+        // so that each second-product operand P^T[ct][s] is complete well before the slot that consumes it.  The thirds
+        // are cut so that their issue times are about equal (a transcendental instruction costs a lone wave about 10
+        // cycles, a plain one about 6): 3 plain + 1 transcendental, 2 + 2, 4 + 1.
+        float t1 = 0, s0 = 0;
         auto chunk = [&](auto c_) {
             constexpr int c = decltype(c_)::value;
             constexpr int pi = c / 3, third = c % 3;
             constexpr int ct = (pi / 4) % 2, pp = (pi % 4) + 4 * (pi / 8), i0 = 2 * pp, i1 = i0 + 1;
             if constexpr (third == 0) {
-                e0 = __builtin_amdgcn_exp2f(-LOG2E * mc[ct][i0]);
-                e1 = __builtin_amdgcn_exp2f(-LOG2E * mc[ct][i1]);
+                const float t0 = -LOG2E * mc[ct][i0];
+                t1 = -LOG2E * mc[ct][i1];
+                e0 = __builtin_amdgcn_exp2f(t0);
                 xn0 = mc[ct][i0] * nc[ct][i0];
             } else if constexpr (third == 1) {
-                e0 = __builtin_amdgcn_rcpf(__builtin_fmaf(e0, rinv[ct], rinv[ct]));
-                e1 = __builtin_amdgcn_rcpf(__builtin_fmaf(e1, rinv[ct], rinv[ct]));
+                e1 = __builtin_amdgcn_exp2f(t1);
+                s0 = __builtin_amdgcn_rcpf(__builtin_fmaf(e0, rinv[ct], rinv[ct]));
                 xn1 = mc[ct][i1] * nc[ct][i1];
             } else {
-                pt[ct][i0 >> 3][i0 & 7] = (bf16_t)(xn0 * e0);
-                pt[ct][i0 >> 3][i1 & 7] = (bf16_t)(xn1 * e1);
+                const float s1 = __builtin_amdgcn_rcpf(__builtin_fmaf(e1, rinv[ct], rinv[ct]));
+                pt[ct][i0 >> 3][i0 & 7] = (bf16_t)(xn0 * s0);
+                pt[ct][i0 >> 3][i1 & 7] = (bf16_t)(xn1 * s1);
             }
         };
 
