@@ -61,14 +61,16 @@ def test_forward_and_backward_match_the_oracle_over_the_sweep(case):
         _check(got.float().cpu(), ref, name, case)
 
 
-# More experts than the 64 whose gate values the forward and the dQ/dR kernel hold in LDS at a time: one expert past a
-# window, exactly two windows, windows that end inside the four-block trips of the forward (d_e = 64: two blocks per
-# expert), three windows with a ragged last one.
+# More experts than the 64 whose gate values the forward and the dQ/dR kernel hold in LDS at a time (the forward restages
+# the tile every 64 experts, the dQ/dR kernel refills it as a ring, 32 slots at a time): one expert past 64, exactly 128,
+# counts that end inside the four-block trips of the forward (d_e = 64: two blocks per expert), 200 with one block per
+# expert, 97 with three.
 CASES_MANY_EXPERTS = [
     (1, 2, 300, 128, 65, 32, 1, False, "bf16"),
     (2, 1, 257, 64, 128, 32, 1, True, "f32"),
     (1, 2, 513, 96, 130, 64, 2, False, "bf16"),
     (1, 1, 64, 128, 200, 32, 1, True, "bf16"),
+    (1, 1, 200, 64, 97, 96, 1, False, "bf16"),       # three blocks per expert, the ring refilled twice
 ]
 
 
