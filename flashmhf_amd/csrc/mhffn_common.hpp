@@ -31,7 +31,9 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // 16-byte cop
 
 constexpr int JB = 32;          // rows of K/U/V per block
 // Experts whose gate values the forward and the dQ/dR kernel keep in LDS at a time ([GATE_WIN][256 tokens] fp32 = 64 KB,
-// next to the 96 KB weight ring); a power of two, and a window is a multiple of four blocks whatever d_e is.
+// next to the 96 KB weight ring); a power of two.  With more experts the forward restages the tile every GATE_WIN experts
+// (a multiple of four blocks whatever d_e is, so every window starts on its LDS stage 0) and the dQ/dR kernel refills it
+// as a ring, expert e in slot e % GATE_WIN.
 constexpr int GATE_WIN = 64;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float FLT_MAX_F = 3.402823466e+38f;
@@ -261,11 +263,6 @@ template <int N>
 __device__ __forceinline__ void lds_wait_n()
 {
     asm volatile("s_waitcnt lgkmcnt(%0)" :: "n"(N));
-}
-template <int N>
-__device__ __forceinline__ void lds_wait_n(u32x4& a, u32x4& b)
-{
-    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
 }
 template <int N>
 __device__ __forceinline__ void lds_wait_n(u32x4& a, u32x4& b, u32x4& c, u32x4& d, u32x4& e, u32x4& f)
